@@ -1,0 +1,133 @@
+/*
+ * w4a16_gfx950.h — C ABI of the MI355X (gfx950) weight-only int4 GEMM library.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the default stream), launches asynchronously on
+ * that stream, never synchronises the host, and returns 0 on success or a
+ * negative W4A16_E* code.  After a failure w4a16_last_error() returns a
+ * message worded like the reference's TORCH_CHECK texts (thread-local).
+ * The caller owns every buffer.  Nothing here allocates device memory.
+ *
+ * Each function names the reference operator it stands in for.
+ */
+#ifndef W4A16_GFX950_H
+#define W4A16_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define W4A16_ABI_VERSION 1
+
+enum {
+  W4A16_OK = 0,
+  W4A16_EINVAL = -1,   /* shape / argument check failed (reference: TORCH_CHECK)     */
+  W4A16_ENOTIMPL = -2, /* valid in the reference, not built here (e.g. 8-bit, fp8)   */
+  W4A16_EHIP = -3      /* a HIP runtime call failed                                  */
+};
+
+/* weight types (decoded from the reference's ScalarType ids by the host layer,
+ * vllm/scalar_type.py:136-164, csrc/core/scalar_type.hpp:143-160) */
+enum { W4A16_WTYPE_U4B8 = 0, W4A16_WTYPE_U4 = 1 };
+/* activation / output / scale element type */
+enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1 };
+
+int w4a16_abi_version(void);
+const char* w4a16_last_error(void);
+
+/* Replaces torch.ops._C.gptq_marlin_repack
+ * (csrc/quantization/gptq_marlin/gptq_marlin_repack.cu:251-322, schema csrc/torch_bindings.cpp:327-329).
+ * b_q_weight: int32 [size_k/8, size_n] GPTQ packing (nibble i of word (r,n) = q[8r+i, n]).
+ * perm: int32 [size_k] source-row order (act-order) or NULL.
+ * out: int32 [size_k/16, 2*size_n] Marlin layout. */
+int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm, uint32_t* out,
+                             int64_t size_k, int64_t size_n, int num_bits, void* stream);
+
+/* Replaces torch.ops._C.awq_marlin_repack
+ * (csrc/quantization/gptq_marlin/awq_marlin_repack.cu:189-248, schema csrc/torch_bindings.cpp:333-335).
+ * b_q_weight: int32 [size_k, size_n/8] AWQ packing (nibble t of word (k,c) = q[k, 8c+{0,2,4,6,1,3,5,7}[t]]). */
+int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
+                            int64_t size_n, int num_bits, void* stream);
+
+/* Replaces torch.ops._C.permute_cols (csrc/permute_cols.cu:14-88, schema csrc/torch_bindings.cpp:312):
+ * out[m, k] = a[m, perm[k]] for 16-bit elements; a has row stride lda (elements), out is dense. */
+int w4a16_permute_cols(const void* a, const int32_t* perm, void* out, int64_t size_m,
+                       int64_t size_k, int64_t lda, void* stream);
+
+/* Operands of one W4A16 GEMM  C[M,N] = A[M,K] * dequant(Bq)[K,N] (+ bias).
+ * Mirrors the tensor arguments of torch.ops._C.gptq_marlin_gemm
+ * (csrc/quantization/gptq_marlin/gptq_marlin.cu:674-959, schema csrc/torch_bindings.cpp:316-323)
+ * and, when the moe_* fields are set, of torch.ops._moe_C.moe_wna16_marlin_gemm
+ * (csrc/moe/marlin_moe_wna16/ops.cu:691-993, schema csrc/moe/torch_bindings.cpp:63-75). */
+typedef struct w4a16_gemm_args {
+  uint32_t struct_size;       /* sizeof(w4a16_gemm_args), checked                         */
+  int32_t dtype;              /* W4A16_DTYPE_*: element type of a, c, b_scales, b_bias    */
+  int32_t wtype;              /* W4A16_WTYPE_*                                            */
+  int32_t flags;              /* W4A16_F_* bits                                           */
+  const void* a;              /* [size_m, size_k], row stride lda elements, 16-B aligned  */
+  int64_t lda;
+  void* c;                    /* [size_m(*top_k), size_n] dense                           */
+  const uint32_t* b_q_weight; /* [E,] [size_k/16, 2*size_n] Marlin layout                 */
+  const void* b_scales;       /* [E,] [num_groups, size_n] Marlin-permuted                */
+  const uint32_t* b_zeros;    /* [E,] [num_groups, size_n/8] Marlin-packed, or NULL       */
+  const int32_t* g_idx;       /* [E,] [size_k] sorted group of each Marlin row, or NULL   */
+  const int32_t* perm;        /* [E,] [size_k] act-order column gather for a, or NULL     */
+  const void* b_bias;         /* [E,] [size_n] Marlin-permuted bias, or NULL              */
+  float* c_tmp;               /* fp32 scratch, >= w4a16_gemm_scratch_bytes(); may be NULL
+                                 when that returns 0                                      */
+  int32_t* workspace;         /* int32 counters, all zero on entry, all zero on exit      */
+  int64_t workspace_len;      /* elements                                                 */
+  int64_t size_m, size_n, size_k;
+  int64_t num_groups;         /* rows of b_scales (per expert)                            */
+  /* ---- fused-MoE variant (all NULL/0 for the dense op) ---- */
+  const int32_t* sorted_token_ids;       /* [n_sorted]  (pad value >= size_m*top_k)       */
+  const int32_t* expert_ids;             /* [ceil(n_sorted/moe_block_size)], -1 = skip    */
+  const int32_t* num_tokens_past_padded; /* [1] device scalar                             */
+  const float* topk_weights;             /* flat, indexed by sorted token id              */
+  int64_t n_sorted;
+  int32_t moe_block_size;     /* 8 or a multiple of 16 in [16, 64]                        */
+  int32_t top_k;
+  int32_t num_experts;
+  int32_t reserved;
+} w4a16_gemm_args;
+
+enum {
+  W4A16_F_IS_K_FULL = 1,        /* act-order: groups are whole on this shard              */
+  W4A16_F_USE_ATOMIC_ADD = 2,   /* accepted; the split-K reduction here is always ordered */
+  W4A16_F_USE_FP32_REDUCE = 4,  /* accepted; partial sums are always fp32                 */
+  W4A16_F_MUL_TOPK_WEIGHTS = 8, /* MoE: scale each output row by its routing weight       */
+  W4A16_F_MOE = 16
+};
+
+/* Bytes of fp32 scratch (c_tmp) a call with these operands may use (0 = none).
+ * The reference allocates the equivalent inside the op (gptq_marlin.cu:751-763). */
+int64_t w4a16_gemm_scratch_bytes(const w4a16_gemm_args* args);
+
+/* Replaces torch.ops._C.gptq_marlin_gemm / torch.ops._moe_C.moe_wna16_marlin_gemm (see above). */
+int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream);
+
+/* Replaces torch.ops._moe_C.moe_align_block_size
+ * (csrc/moe/moe_align_sum_kernels.cu:275-346, schema csrc/moe/torch_bindings.cpp:17-23).
+ * topk_ids int32 [numel]; sorted_token_ids int32 [sorted_len] (pre-filled with numel by this call);
+ * expert_ids int32 [expert_ids_len] (tail zero-filled); num_tokens_post_pad int32 [1]. */
+int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int32_t num_experts,
+                               int32_t block_size, int32_t* sorted_token_ids, int64_t sorted_len,
+                               int32_t* expert_ids, int64_t expert_ids_len,
+                               int32_t* num_tokens_post_pad, void* stream);
+
+/* Replaces torch.ops._moe_C.moe_sum (csrc/moe/moe_align_sum_kernels.cu:375-416, schema
+ * csrc/moe/torch_bindings.cpp:13): out[t, :] = sum_k in[t, k, :], 16-bit elements, fp32 sum. */
+int w4a16_moe_sum(const void* in, void* out, int64_t tokens, int32_t top_k, int64_t hidden,
+                  int32_t dtype, void* stream);
+
+/* Replaces torch.ops._C.silu_and_mul (csrc/activation_kernels.cu:22-32,85; schema
+ * csrc/torch_bindings.cpp:118): out[t, j] = silu(in[t, j]) * in[t, d + j]. */
+int w4a16_silu_and_mul(const void* in, void* out, int64_t tokens, int64_t d, int32_t dtype,
+                       void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A16_GFX950_H */

@@ -1,0 +1,91 @@
+"""Dequantize-then-matmul reference for the W4A16 GEMM (CPU oracle, test infrastructure only).
+
+The reference's kernel test (tests/kernels/quantization/test_marlin_gemm.py:228-361)
+checks `gptq_marlin_gemm` against `torch.matmul(a, w_ref)` where `w_ref` is the
+dequantised weight produced by the quantizer (quant_utils.py:427-432:
+w_ref = (q - zp) * s in the weight dtype).  Here the same thing is computed from the
+tensors the op actually receives, so layout decode, scale/zero indexing and act-order
+are all part of what is checked:
+
+  dequant_marlin(...)   Marlin-layout operands  -> w [K, N] in the activation dtype
+  dequant_checkpoint()  GPTQ / AWQ checkpoint   -> w [K, N]   (the CPU baseline path:
+                        unpack nibbles, (q-8)*s or (q-z)*s group-broadcast)
+  gemm_ref(a, w)        fp32 matmul (+ bias), result in fp32
+
+Pinned by (tests/test_oracle_gemm.py): dequant_marlin(repack(x)) == w_ref of the
+quantizer bit-for-bit for every (type, group, act-order) combination;
+dequant_checkpoint == w_ref likewise; fp32 matmul is torch's.
+"""
+import numpy as np
+import torch
+
+from .marlin_layout import (marlin_unpack_weights, marlin_unpack_zero_points,
+                            marlin_unpermute_scales)
+from .quant_utils import awq_unpack, unpack_rows
+
+
+def _expand_groups(t: torch.Tensor, size_k: int, g_idx=None) -> torch.Tensor:
+    """[G, N] -> [K, N] by group broadcast (contiguous groups) or g_idx lookup."""
+    g = t.shape[0]
+    if g_idx is not None and len(g_idx) > 0:
+        return t[g_idx.long()]
+    if g == 1:
+        return t.expand(size_k, -1)
+    assert size_k % g == 0
+    return t.repeat_interleave(size_k // g, dim=0)
+
+
+def dequant_marlin(b_q_weight, b_scales, b_zeros, g_idx, size_k, size_n, bias8: bool, dtype):
+    """Marlin operands -> dense w[K, N] (row i = Marlin row i, i.e. after act-order sort).
+
+    b_scales [G, N] Marlin-permuted; b_zeros int32 [G, N/8] Marlin-packed or None;
+    g_idx: sorted group id per Marlin row (only when the scale row is looked up per row).
+    """
+    q = marlin_unpack_weights(b_q_weight)
+    assert tuple(q.shape) == (size_k, size_n)
+    num_groups = b_scales.shape[0]
+    grouped = num_groups > 1
+    s = marlin_unpermute_scales(b_scales, grouped).to(dtype)
+    s_full = _expand_groups(s, size_k, g_idx)
+    if b_zeros is not None and b_zeros.numel() > 0:
+        z = marlin_unpack_zero_points(b_zeros)
+        z_full = _expand_groups(z, size_k, g_idx)
+        qz = q - z_full
+    else:
+        qz = q - (8 if bias8 else 0)
+    return qz.to(dtype) * s_full
+
+
+def dequant_checkpoint(qweight, scales, qzeros, g_idx, fmt: str, dtype):
+    """Checkpoint tensors -> dense w[K, N] in original row order.
+
+    fmt "gptq": qweight int32 [K/8, N], symmetric uint4b8 (qzeros ignored), g_idx optional.
+    fmt "awq":  qweight int32 [K, N/8], qzeros int32 [G, N/8] (AWQ interleave), scales [G, N].
+    """
+    if fmt == "gptq":
+        q = unpack_rows(qweight, 4) - 8
+    elif fmt == "awq":
+        q = awq_unpack(qweight, 4)
+    else:
+        raise ValueError(fmt)
+    k = q.shape[0]
+    s_full = _expand_groups(scales.to(dtype), k, g_idx)
+    if fmt == "awq":
+        q = q - _expand_groups(awq_unpack(qzeros, 4), k, g_idx)
+    return q.to(dtype) * s_full
+
+
+def gemm_ref(a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    out = a.float() @ w.float()
+    if bias is not None:
+        out = out + bias.float()
+    return out
+
+
+def error_metrics(out: torch.Tensor, ref: torch.Tensor) -> dict:
+    """max|d|/max|ref| (the stated 2e-2 / 4e-2 gate) and the reference test's
+    mean|d|/mean|ref| (< 0.04, test_marlin_gemm.py:78-81)."""
+    d = (out.float().cpu() - ref.float().cpu()).abs()
+    r = ref.float().cpu().abs()
+    return {"max_rel": float(d.max() / r.max().clamp(min=1e-30)),
+            "mean_rel": float(d.mean() / r.mean().clamp(min=1e-30))}

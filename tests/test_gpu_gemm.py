@@ -1,0 +1,174 @@
+"""GPU parity of the W4A16 GEMM against the CPU oracle (dequantize, fp32 matmul), through the torch
+op -> C ABI -> HIP kernels.  Tolerances: max|out-ref|/max|ref| <= 2e-2 (fp16) / 4e-2 (bf16) and the
+reference test's mean|out-ref|/mean|ref| < 0.04 (tests/kernels/quantization/test_marlin_gemm.py:78-81,
+359-361); one-hot activations must reproduce the dequantised weight rows bit-for-bit."""
+import pytest
+import torch
+
+from helpers import check_close, make_layer, run_gemm
+from oracle import gemm_ref as gr
+
+pytestmark = pytest.mark.gpu
+
+MNK_FACTORS = [(1, 1, 1), (1, 4, 8), (26, 37, 13), (257, 13, 11)]
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    import vllm_amd.ops as o
+    return o
+
+
+@pytest.fixture(scope="module")
+def workspace(dev):
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    return marlin_make_workspace_new(dev)
+
+
+def _a(m, k, dtype, dev, seed=11):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(m, k, generator=g).to(dtype).to(dev)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("has_zp", [False, True])
+@pytest.mark.parametrize("group_size", [-1, 32, 64, 128])
+def test_one_hot_rows_are_exact(ops, dev, workspace, dtype, has_zp, group_size):
+    """A = unit vectors: every output row is a single product 1 * w, so it must equal w_ref exactly.
+    Pins layout decode, nibble order, the -8 bias / zero points and scale indexing with zero tolerance."""
+    size_k, size_n = 512, 320
+    print(f"one_hot dtype={dtype} zp={has_zp} g={group_size}", flush=True)
+    layer = make_layer(size_k, size_n, group_size, dtype, has_zp=has_zp, seed=5)
+    ks = torch.tensor([0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 100, 127, 128, 300, 511])
+    a = torch.zeros(16, size_k, dtype=dtype)
+    a[torch.arange(16), ks] = 1.0
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_one_hot_every_k(ops, dev, workspace, dtype):
+    """All K positions of a 256-deep layer, 64 rows at a time (also exercises the 4-m-block tile)."""
+    size_k, size_n = 256, 128
+    layer = make_layer(size_k, size_n, 64, dtype, seed=6)
+    a = torch.eye(size_k, dtype=dtype)
+    for m0 in range(0, size_k, 64):
+        print(f"one_hot_all dtype={dtype} rows={m0}", flush=True)
+        out = run_gemm(ops, layer, a[m0:m0 + 64].contiguous().to(dev), dev, workspace)
+        assert torch.equal(out.cpu(), layer.w_ref[m0:m0 + 64])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("is_k_full", [True, False])
+def test_one_hot_act_order(ops, dev, workspace, dtype, is_k_full):
+    size_k, size_n = 512, 192
+    print(f"one_hot_act_order dtype={dtype} k_full={is_k_full}", flush=True)
+    layer = make_layer(size_k, size_n, 64, dtype, act_order=True, seed=8)
+    ks = torch.randperm(size_k, generator=torch.Generator().manual_seed(2))[:32]
+    a = torch.zeros(32, size_k, dtype=dtype)
+    a[torch.arange(32), ks] = 1.0
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace, is_k_full=is_k_full)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n_chunk", [64, 256])
+@pytest.mark.parametrize("mnk", MNK_FACTORS)
+@pytest.mark.parametrize("group_size", [-1, 32, 64, 128])
+@pytest.mark.parametrize("mode", ["gptq", "gptq_act_order", "gptq_act_order_partial_k", "awq"])
+def test_gemm_reference_grid(ops, dev, workspace, dtype, n_chunk, mnk, group_size, mode):
+    """The reference's test_gptq_marlin_gemm grid restricted to the 4-bit types."""
+    mf, nf, kf = mnk
+    size_m, size_k, size_n = mf, 128 * kf, n_chunk * nf
+    act_order = mode.startswith("gptq_act_order")
+    if act_order and (group_size == -1 or group_size == size_k):
+        pytest.skip("act-order needs more than one group")
+    if size_k % (group_size if group_size > 0 else size_k) != 0:
+        pytest.skip("group does not divide K")
+    print(f"grid {mode} dtype={dtype} m={size_m} n={size_n} k={size_k} g={group_size}", flush=True)
+    layer = make_layer(size_k, size_n, group_size, dtype, has_zp=(mode == "awq"), act_order=act_order,
+                       seed=size_n + size_k)
+    a = _a(size_m, size_k, dtype, dev)
+    out = run_gemm(ops, layer, a, dev, workspace, is_k_full=(mode != "gptq_act_order_partial_k"))
+    assert out.shape == (size_m, size_n) and out.dtype == dtype
+    check_close(out, a, layer)
+    assert int(workspace.abs().sum()) == 0
+
+
+def test_integer_exact(ops, dev, workspace):
+    """Unit scales and small-integer activations: every partial sum is an exact integer below 2^24,
+    so the GEMM must equal the integer matmul exactly whatever the summation order."""
+    size_m, size_k, size_n = 48, 1024, 256
+    g = torch.Generator().manual_seed(4)
+    layer = make_layer(size_k, size_n, 128, torch.float16, seed=9)
+    layer.marlin_s = torch.ones_like(layer.marlin_s)
+    a = torch.randint(-4, 5, (size_m, size_k), generator=g).half()
+    want = a.float() @ (layer.q.float() - 8)
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    assert torch.equal(out.float().cpu(), want.half().float())
+
+
+def test_rows_independent_of_m_and_deterministic(ops, dev, workspace):
+    """Row m of the result does not depend on M, on the other rows, or on the run (ordered split-K)."""
+    size_k, size_n = 4096, 1024
+    layer = make_layer(size_k, size_n, 128, torch.float16, seed=10, w_std=0.02)
+    a = _a(200, size_k, torch.float16, dev)
+    full = run_gemm(ops, layer, a, dev, workspace)
+    again = run_gemm(ops, layer, a, dev, workspace)
+    assert torch.equal(full, again)
+    for m in (1, 4, 16, 17, 64, 65):
+        part = run_gemm(ops, layer, a[:m].contiguous(), dev, workspace)
+        d = (part.float() - full[:m].float()).abs().max() / full.float().abs().max()
+        assert float(d) < 2e-3, (m, float(d))   # same operands, only the split-K partition may differ
+    assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_strided_a_and_bias_and_given_c(ops, dev, workspace, dtype):
+    """Sub-view activations (test_marlin_gemm.py:537-581), bias (:584-629), caller-provided output."""
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    size_m, size_k, size_n = 37, 512, 384
+    layer = make_layer(size_k, size_n, 128, dtype, seed=12)
+    g = torch.Generator().manual_seed(13)
+    big = torch.randn(size_m, size_k + 64, generator=g).to(dtype).to(dev)
+    a = big[:, 32:32 + size_k]
+    assert not a.is_contiguous()
+    bias = torch.randn(size_n, generator=g).to(dtype).to(dev)
+    c = torch.empty(size_m, size_n, dtype=dtype, device=dev)
+    out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias), c=c)
+    assert out.data_ptr() == c.data_ptr()
+    check_close(out, a, layer, bias=bias)
+
+
+def test_empty_m(ops, dev, workspace):
+    layer = make_layer(128, 64, 128, torch.float16)
+    out = run_gemm(ops, layer, torch.empty(0, 128, dtype=torch.float16, device=dev), dev, workspace)
+    assert out.shape == (0, 64)
+
+
+def test_argument_errors(ops, dev, workspace):
+    layer = make_layer(128, 64, 128, torch.float16)
+    a = torch.zeros(4, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError):
+        run_gemm(ops, layer, torch.zeros(4, 64, dtype=torch.float16, device=dev), dev, workspace)   # K mismatch
+    with pytest.raises(RuntimeError):
+        run_gemm(ops, layer, a.float(), dev, workspace)                                              # dtype
+    import vllm_amd.scalar_type as vst
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ops.gptq_marlin_gemm(a, None, layer.marlin_q.to(dev), None, layer.marlin_s.to(dev), None, None, None, None,
+                             workspace, vst.scalar_types.uint8b128, 4, 64, 128)
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (4096, 6144), (14336, 4096)])
+@pytest.mark.parametrize("m", [1, 16, 64, 256])
+def test_llama_shapes_fp16(ops, dev, workspace, shape, m):
+    """Configuration 1 / 2 shapes: N(0,1) activations, N(0, 0.02) weights, absmax/7 RTN, group 128."""
+    size_k, size_n = shape
+    print(f"llama k={size_k} n={size_n} m={m}", flush=True)
+    layer = make_layer(size_k, size_n, 128, torch.float16, seed=1, w_std=0.02, rule="benchmark")
+    a = _a(m, size_k, torch.float16, dev, seed=2)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    assert int(workspace.abs().sum()) == 0

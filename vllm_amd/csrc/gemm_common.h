@@ -1,0 +1,158 @@
+// Device-side building blocks shared by the W4A16 GEMM kernels (gfx950, wave64).
+//
+// How a wavefront consumes the Marlin weight layout with v_mfma_f32_16x16x32_{f16,bf16}
+// -----------------------------------------------------------------------------------
+// Lane l is split as c = l & 7, h = (l >> 3) & 1, g = l >> 4.  For a "column pair" cp (two
+// adjacent 64-column n-tiles, 128 columns) and a k-step ks (two adjacent 16-row k-tiles, 32 rows)
+// the lane issues two 128-bit loads, one per k-tile, at Marlin word
+//     kt*2N + (2cp+h)*128 + (4c+g)*4 ,  kt = 2ks, 2ks+1
+// i.e. it plays Marlin "thread" th = 4c+g of n-tile 2cp+h.  The 64 lanes of one load cover one
+// contiguous KiB.  Word w (0..3) of a load holds rows {2g, 2g+1, 2g+8, 2g+9} of the k-tile for
+// columns n0 = 64(2cp+h) + 16w + c and n0 + 8.  Across the two k-tiles the lane therefore owns,
+// for each of its 8 columns, the 8 K-rows  {2g, 2g+1, 2g+8, 2g+9, 16+2g, 16+2g+1, 16+2g+8, 16+2g+9}
+// — exactly what one lane of the MFMA's 32x16 B operand holds (column label l & 15, K-block
+// l >> 4).  So 8 MFMAs per k-step, one per (w, half), each covering the 16 columns
+//     { 64(2cp+h) + 16w + 8half + c : h in {0,1}, c in [0,8) }      (label = 8h + c)
+// K order inside the MFMA is arbitrary as long as the activation operand agrees: activations are
+// staged in LDS as [k-step][g][row m][8 halves in the K order above], so lane (m = l & 15,
+// g = l >> 4) fetches its A operand with one conflict-free ds_read_b128.
+// The accumulator of lane l holds rows 4(l>>4) .. +3 of column label l & 15 — the lane's own
+// columns, so per-column scales / zero-points / bias never cross lanes.
+#pragma once
+#include "common.h"
+
+namespace w4a16 {
+
+using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+using u32x2 = uint32_t __attribute__((ext_vector_type(2)));
+using f32x4 = float __attribute__((ext_vector_type(4)));
+using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
+using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+
+enum { DT_F16 = 0, DT_BF16 = 1 };
+// how the scale row of a K-row is found
+enum {
+  GM_GROUPED = 0,  // contiguous groups of group_size rows (multiple of 32), scale per element
+  GM_CHANNEL = 1,  // one scale row for all K: applied once to the fp32 accumulator
+  GM_GIDX = 2      // scale row = g_idx[row] (act-order shard with partial groups)
+};
+
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16x16x32(u32x4 a, u32x4 b, f32x4 c) {
+  if constexpr (DT == DT_F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f16x2 as_h2(uint32_t x) { return __builtin_bit_cast(f16x2, x); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ float bf16_lo_f32(uint32_t x) { return __builtin_bit_cast(float, x << 16); }
+__device__ __forceinline__ float bf16_hi_f32(uint32_t x) { return __builtin_bit_cast(float, x & 0xffff0000u); }
+__device__ __forceinline__ float f16_lo_f32(uint32_t x) { return (float)as_h2(x).x; }
+__device__ __forceinline__ float f16_hi_f32(uint32_t x) { return (float)as_h2(x).y; }
+
+// round-to-nearest-even pack of two fp32 into bf16x2 (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  bf2 r = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  f16x2 r = {(_Float16)lo, (_Float16)hi};
+  return as_u32(r);
+}
+
+// Per-lane dequantisation constants of one Marlin word position w (two columns: half 0 / half 1).
+//  fp16:  value = (1024+q) - zl  |  (1024+16q)/16 - zh , then * s         (all packed-half ops;
+//         every step is exact except the final multiply, so the operand equals
+//         half(q - z) * half(s) rounded once — the reference's w_ref)
+//  bf16:  value = bf16_rne( fma(float(q), s, c) ),  c = -z*s exact in fp32  (single rounding)
+template <int DT>
+struct ColConst;
+
+template <>
+struct ColConst<DT_F16> {
+  uint32_t s;   // (s_half0, s_half1)
+  uint32_t zl;  // (1024+z_half0, 1024+z_half1)
+  uint32_t zh;  // (64+z_half0, 64+z_half1)
+};
+template <>
+struct ColConst<DT_BF16> {
+  float s0, s1;  // scale of half 0 / half 1
+  float c0, c1;  // -z*s
+};
+
+// raw: (s_half0, s_half1) packed 16-bit pair as loaded; z0/z1: integer zero points (8 for uint4b8)
+template <int DT, bool UNIT_SCALE>
+__device__ __forceinline__ ColConst<DT> make_col_const(uint32_t s_pair, uint32_t z0, uint32_t z1) {
+  ColConst<DT> cc;
+  if constexpr (DT == DT_F16) {
+    cc.s = UNIT_SCALE ? 0x3c003c00u : s_pair;
+    // 1024+z and 64+z are exact fp16 integers: 0x6400 | z  and  0x5400 + (z << 4) (ulp of 64.. is 1/16)
+    cc.zl = 0x64006400u | z0 | (z1 << 16);
+    cc.zh = 0x54005400u + ((z0 << 4) | (z1 << 20));
+  } else {
+    cc.s0 = UNIT_SCALE ? 1.0f : bf16_lo_f32(s_pair);
+    cc.s1 = UNIT_SCALE ? 1.0f : bf16_hi_f32(s_pair);
+    cc.c0 = -(float)z0 * cc.s0;
+    cc.c1 = -(float)z1 * cc.s1;
+  }
+  return cc;
+}
+
+// xa, xb: word w of the lane's 128-bit loads from k-tile 2ks and 2ks+1.
+// o0 / o1: MFMA B operand (8 values in the lane's K order) for column half 0 / half 1.
+template <int DT, bool UNIT_SCALE>
+__device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const ColConst<DT>& cc, u32x4& o0,
+                                             u32x4& o1) {
+  if constexpr (DT == DT_F16) {
+    const uint32_t MLO = 0x000f000fu, MHI = 0x00f000f0u, EX = 0x64006400u;
+    const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const f16x2 s = as_h2(cc.s), zl = as_h2(cc.zl), zh = as_h2(cc.zh);
+    const f16x2 s0 = {s.x, s.x}, s1 = {s.y, s.y};
+    const f16x2 zl0 = {zl.x, zl.x}, zl1 = {zl.y, zl.y};
+    const f16x2 zh0 = {zh.x, zh.x}, zh1 = {zh.y, zh.y};
+    auto lo = [&](uint32_t x, f16x2 z, f16x2 sc) {
+      const f16x2 v = as_h2((x & MLO) | EX) - z;
+      return as_u32(UNIT_SCALE ? v : v * sc);
+    };
+    auto hi = [&](uint32_t x, f16x2 z, f16x2 sc) {
+      const f16x2 v = as_h2((x & MHI) | EX) * sixteenth - z;
+      return as_u32(UNIT_SCALE ? v : v * sc);
+    };
+    const uint32_t ya = xa >> 8, yb = xb >> 8;
+    o0 = u32x4{lo(xa, zl0, s0), hi(xa, zh0, s0), lo(xb, zl0, s0), hi(xb, zh0, s0)};
+    o1 = u32x4{lo(ya, zl1, s1), hi(ya, zh1, s1), lo(yb, zl1, s1), hi(yb, zh1, s1)};
+  } else {
+    // nibble j of a word: j=0 (k0,n0) 1 (k0+8,n0) 2 (k0,n0+8) 3 (k0+8,n0+8) 4..7 same with k0+1
+    auto cvt = [&](uint32_t x, uint32_t& a0, uint32_t& a1, uint32_t& b0, uint32_t& b1) {
+      const uint32_t e = x & 0x0f0f0f0fu;         // bytes: nibbles 0,2,4,6
+      const uint32_t o = (x >> 4) & 0x0f0f0f0fu;  // bytes: nibbles 1,3,5,7
+      const float n0 = (float)(e & 0xff), n2 = (float)((e >> 8) & 0xff), n4 = (float)((e >> 16) & 0xff),
+                  n6 = (float)(e >> 24);
+      const float n1 = (float)(o & 0xff), n3 = (float)((o >> 8) & 0xff), n5 = (float)((o >> 16) & 0xff),
+                  n7 = (float)(o >> 24);
+      a0 = pack_bf16(__builtin_fmaf(n0, cc.s0, cc.c0), __builtin_fmaf(n4, cc.s0, cc.c0));  // (k0,k0+1) half0
+      a1 = pack_bf16(__builtin_fmaf(n1, cc.s0, cc.c0), __builtin_fmaf(n5, cc.s0, cc.c0));  // (k0+8,k0+9) half0
+      b0 = pack_bf16(__builtin_fmaf(n2, cc.s1, cc.c1), __builtin_fmaf(n6, cc.s1, cc.c1));
+      b1 = pack_bf16(__builtin_fmaf(n3, cc.s1, cc.c1), __builtin_fmaf(n7, cc.s1, cc.c1));
+    };
+    uint32_t p0, p1, p2, p3, q0, q1, q2, q3;
+    cvt(xa, p0, p1, q0, q1);
+    cvt(xb, p2, p3, q2, q3);
+    o0 = u32x4{p0, p1, p2, p3};
+    o1 = u32x4{q0, q1, q2, q3};
+  }
+}
+
+// Position of real column `cl` (0..31 inside its 32-column chunk) in a tensor permuted with the
+// reference's "single" permutation (marlin_utils.py:278-286, used for channel-wise scales and bias).
+__device__ __forceinline__ int single_perm_pos(int cl) {
+  return 8 * ((cl & 7) >> 1) + 2 * (cl >> 3) + (cl & 1);
+}
+
+}  // namespace w4a16

@@ -1,0 +1,20 @@
+// Launch plan shared between the host entry point and the kernel launchers.
+#pragma once
+#include "gemm_common.h"
+
+namespace w4a16 {
+
+struct Plan {
+  int gm;            // GM_*: how scale rows are found
+  int group_ksteps;  // GM_GROUPED: group_size / 32
+  bool use_perm;     // gather A columns through perm (act-order)
+  int mb, bm;        // m-blocks of 16 rows per tile, rows per tile
+  int mtiles, ncp, tiles;
+  int total_ksteps, splits, kps;  // k-steps of 32 rows; K splits; k-steps per split
+  int xcd_map;
+  int64_t ctmp_bytes;
+};
+
+int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
+
+}  // namespace w4a16

@@ -1,0 +1,192 @@
+// MoE glue kernels for gfx950: token->expert block alignment, top-k sum, SiLU-and-mul.
+//
+// moe_align_block_size follows the contract of the reference op
+// (vllm/model_executor/layers/fused_moe/moe_align_block_size.py:11-85, kernels
+// csrc/moe/moe_align_sum_kernels.cu:83-268): sort the flattened (token, slot) indices by expert,
+// pad every expert's run to a multiple of block_size with the value `numel`, emit one expert id
+// per block (tail zero-filled) and the padded total.  Unlike the reference (atomic ranks, order
+// inside an expert unspecified) the order here is stable — ascending flat index inside each
+// expert — so the result is deterministic and equals the reference's torch golden
+// (tests/kernels/moe/test_moe_align_block_size.py:92-168) element for element.
+#include "gemm_common.h"
+
+namespace w4a16 {
+
+constexpr int ALIGN_THREADS = 1024;
+constexpr int ALIGN_WAVES = ALIGN_THREADS / 64;
+constexpr int ALIGN_MAX_EXPERTS = 1024;
+
+// Every workgroup recomputes the histogram and the scan (numel and E are small), then its 16
+// wavefronts each place the tokens of experts wg*16 + wave, +gridDim*16, ... by ballot ranking.
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(
+    const int32_t* __restrict__ topk_ids, int numel, int num_experts, int block_size,
+    int32_t* __restrict__ sorted_ids, int sorted_len, int32_t* __restrict__ expert_ids, int expert_ids_len,
+    int32_t* __restrict__ num_post_pad) {
+  __shared__ int cnt[ALIGN_MAX_EXPERTS];
+  __shared__ int off[ALIGN_MAX_EXPERTS + 1];
+  const int t = threadIdx.x;
+  for (int e = t; e < num_experts; e += ALIGN_THREADS) cnt[e] = 0;
+  __syncthreads();
+  for (int i = t; i < numel; i += ALIGN_THREADS) {
+    const int e = topk_ids[i];
+    if (e >= 0 && e < num_experts) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (t < 64) {  // wave 0: exclusive scan of padded counts, 64 experts per round
+    int run = 0;
+    for (int base = 0; base < num_experts; base += 64) {
+      const int e = base + t;
+      const int padded = e < num_experts ? (cnt[e] + block_size - 1) / block_size * block_size : 0;
+      int incl = padded;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_up(incl, d, 64);
+        if (t >= d) incl += v;
+      }
+      if (e < num_experts) off[e] = run + incl - padded;
+      run += __shfl(incl, 63, 64);
+    }
+    if (t == 0) off[num_experts] = run;
+  }
+  __syncthreads();
+  const int total = off[num_experts];
+
+  if (blockIdx.x == 0) {
+    if (t == 0) *num_post_pad = total;
+    // expert id of every block; blocks past the padded total are zero-filled
+    for (int e = t; e < num_experts; e += ALIGN_THREADS) {
+      const int b0 = off[e] / block_size, b1 = off[e + 1] / block_size;
+      for (int b = b0; b < b1 && b < expert_ids_len; ++b) expert_ids[b] = e;
+    }
+    for (int b = total / block_size + t; b < expert_ids_len; b += ALIGN_THREADS) expert_ids[b] = 0;
+    for (int i = total + t; i < sorted_len; i += ALIGN_THREADS) sorted_ids[i] = numel;
+  }
+
+  const int lane = t & 63, wv = t >> 6;
+  for (int e = blockIdx.x * ALIGN_WAVES + wv; e < num_experts; e += gridDim.x * ALIGN_WAVES) {
+    int pos = off[e];
+    const int end = off[e + 1];
+    if (pos == end) continue;
+    for (int base = 0; base < numel; base += 64) {
+      const int i = base + lane;
+      const bool hit = i < numel && topk_ids[i] == e;
+      const unsigned long long m = __ballot(hit);
+      if (hit) {
+        const int rank = __popcll(m & ((1ull << lane) - 1ull));
+        if (pos + rank < sorted_len) sorted_ids[pos + rank] = i;
+      }
+      pos += __popcll(m);
+    }
+    for (int i = pos + lane; i < end && i < sorted_len; i += 64) sorted_ids[i] = numel;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
+                                                      int64_t total8, int top_k, int64_t hidden8) {
+  // one thread per 8 consecutive output elements
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total8; idx += (int64_t)gridDim.x * 256) {
+    const int64_t tok = idx / hidden8, col = idx % hidden8;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < top_k; ++k) {
+      const u32x4 v = *(const u32x4*)(in + ((tok * top_k + k) * hidden8 + col) * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[2 * j] += DT == DT_F16 ? f16_lo_f32(v[j]) : bf16_lo_f32(v[j]);
+        acc[2 * j + 1] += DT == DT_F16 ? f16_hi_f32(v[j]) : bf16_hi_f32(v[j]);
+      }
+    }
+    u32x4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      o[j] = DT == DT_F16 ? pack_f16(acc[2 * j], acc[2 * j + 1]) : pack_bf16(acc[2 * j], acc[2 * j + 1]);
+    *(u32x4*)(out + idx * 8) = o;
+  }
+}
+
+// out = T(silu_f32(x)) * y evaluated like the reference's act_and_mul_kernel<silu>
+// (csrc/activation_kernels.cu:22-40): SiLU in fp32 rounded to T, then one multiply rounded to T.
+template <int DT>
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ in,
+                                                           uint16_t* __restrict__ out, int64_t total8,
+                                                           int64_t d8) {
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total8; idx += (int64_t)gridDim.x * 256) {
+    const int64_t tok = idx / d8, col = idx % d8;
+    const u32x4 x = *(const u32x4*)(in + (tok * 2 * d8 + col) * 8);
+    const u32x4 y = *(const u32x4*)(in + (tok * 2 * d8 + d8 + col) * 8);
+    u32x4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float xv[2], yv[2], r[2];
+      xv[0] = DT == DT_F16 ? f16_lo_f32(x[j]) : bf16_lo_f32(x[j]);
+      xv[1] = DT == DT_F16 ? f16_hi_f32(x[j]) : bf16_hi_f32(x[j]);
+      yv[0] = DT == DT_F16 ? f16_lo_f32(y[j]) : bf16_lo_f32(y[j]);
+      yv[1] = DT == DT_F16 ? f16_hi_f32(y[j]) : bf16_hi_f32(y[j]);
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const float s = xv[q] / (1.0f + expf(-xv[q]));
+        const uint32_t sr = DT == DT_F16 ? pack_f16(s, 0.f) : pack_bf16(s, 0.f);
+        const float st = DT == DT_F16 ? f16_lo_f32(sr) : bf16_lo_f32(sr);
+        r[q] = st * yv[q];
+      }
+      o[j] = DT == DT_F16 ? pack_f16(r[0], r[1]) : pack_bf16(r[0], r[1]);
+    }
+    *(u32x4*)(out + idx * 8) = o;
+  }
+}
+
+}  // namespace w4a16
+
+using namespace w4a16;
+
+extern "C" int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int32_t num_experts,
+                                          int32_t block_size, int32_t* sorted_token_ids, int64_t sorted_len,
+                                          int32_t* expert_ids, int64_t expert_ids_len,
+                                          int32_t* num_tokens_post_pad, void* stream) {
+  W4A16_CHECK(topk_ids && sorted_token_ids && expert_ids && num_tokens_post_pad, "null pointer");
+  W4A16_CHECK(num_experts >= 1 && num_experts <= ALIGN_MAX_EXPERTS, "num_experts = %d must be in [1, %d]",
+              num_experts, ALIGN_MAX_EXPERTS);
+  W4A16_CHECK(block_size >= 1, "block_size must be positive");
+  W4A16_CHECK(numel >= 0 && numel < (1LL << 30), "bad topk_ids.numel()");
+  W4A16_CHECK(sorted_len >= numel, "sorted_token_ids is shorter than topk_ids");
+  const int grid = (int)ceil_div(num_experts, ALIGN_WAVES);
+  moe_align_kernel<<<grid, ALIGN_THREADS, 0, (hipStream_t)stream>>>(
+      topk_ids, (int)numel, num_experts, block_size, sorted_token_ids, (int)sorted_len, expert_ids,
+      (int)expert_ids_len, num_tokens_post_pad);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_moe_sum(const void* in, void* out, int64_t tokens, int32_t top_k, int64_t hidden,
+                             int32_t dtype, void* stream) {
+  W4A16_CHECK(in && out, "null pointer");
+  W4A16_CHECK(hidden % 8 == 0, "hidden = %lld must be divisible by 8", (long long)hidden);
+  W4A16_CHECK(dtype == W4A16_DTYPE_F16 || dtype == W4A16_DTYPE_BF16, "unsupported dtype");
+  const int64_t total8 = tokens * (hidden / 8);
+  if (total8 == 0) return 0;
+  const int64_t blocks = ceil_div(total8, 256);
+  const unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
+  if (dtype == W4A16_DTYPE_F16)
+    moe_sum_kernel<DT_F16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, top_k, hidden / 8);
+  else
+    moe_sum_kernel<DT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, top_k, hidden / 8);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_silu_and_mul(const void* in, void* out, int64_t tokens, int64_t d, int32_t dtype,
+                                  void* stream) {
+  W4A16_CHECK(in && out, "null pointer");
+  W4A16_CHECK(d % 8 == 0, "d = %lld must be divisible by 8", (long long)d);
+  W4A16_CHECK(dtype == W4A16_DTYPE_F16 || dtype == W4A16_DTYPE_BF16, "unsupported dtype");
+  const int64_t total8 = tokens * (d / 8);
+  if (total8 == 0) return 0;
+  const int64_t blocks = ceil_div(total8, 256);
+  const unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
+  if (dtype == W4A16_DTYPE_F16)
+    silu_and_mul_kernel<DT_F16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, d / 8);
+  else
+    silu_and_mul_kernel<DT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, d / 8);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}

@@ -1,0 +1,175 @@
+// Checkpoint -> Marlin-layout repack kernels (4-bit), written for gfx950.
+//
+// Output layout (int32 [K/16, 2N]): for k-tile kt (16 rows) and n-tile nt (64 cols) the 128
+// words nt*128 + th*4 + w (th in [0,32), w in [0,4)) hold, with r = 2*(th%4), c = th/4,
+// n0 = 64*nt + 16*w + c, k0 = 16*kt + r, the nibbles
+//   j:   0        1        2          3          4        5        6          7
+//   q[k0,n0] q[k0+8,n0] q[k0,n0+8] q[k0+8,n0+8] q[k0+1,n0] q[k0+9,n0] q[k0+1,n0+8] q[k0+9,n0+8]
+// which is the layout produced by the reference's gptq_marlin_repack / awq_marlin_repack
+// (csrc/quantization/gptq_marlin/gptq_marlin_repack.cu:107-204, awq_marlin_repack.cu:68-148)
+// and by its numpy statement (marlin_utils_test.py:32-93).
+//
+// One workgroup of 256 threads produces the 256 output words of (one k-tile) x (two n-tiles,
+// 128 columns).  The source words of that 16 x 128 patch are staged in LDS with coalesced
+// loads, then each thread assembles one output word, so global reads and writes are both
+// contiguous per wavefront.  The work is pure HBM streaming: K*N/2 bytes in, K*N/2 bytes out.
+#include "common.h"
+
+namespace w4a16 {
+
+// nibble j of the output word takes source row k0 + DK[j], column n0 + DN[j]
+__device__ __constant__ const int kDK[8] = {0, 8, 0, 8, 1, 9, 1, 9};
+
+// GPTQ source: word (r, n), nibble i = q[8r + i, n].  Without perm a k-tile is two source rows.
+template <bool HAS_PERM>
+__global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __restrict__ in,
+                                                          const int32_t* __restrict__ perm,
+                                                          uint32_t* __restrict__ out, int size_k,
+                                                          int size_n) {
+  // LDS: 16 logical rows x 128 columns of source words (HAS_PERM) or 2 x 128 (plain).
+  __shared__ uint32_t tile[HAS_PERM ? 16 : 2][128];
+  __shared__ int src_row[16];
+  const int t = threadIdx.x;
+  const int kt = blockIdx.y;
+  const int ncol0 = blockIdx.x * 128;
+  const int ncols = min(128, size_n - ncol0);  // 64 or 128
+
+  if (HAS_PERM) {
+    if (t < 16) src_row[t] = perm[kt * 16 + t];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = i * 2 + (t >> 7);
+      const int col = t & 127;
+      if (col < ncols) tile[row][col] = in[(size_t)(src_row[row] >> 3) * size_n + ncol0 + col];
+    }
+  } else {
+    const int row = t >> 7, col = t & 127;
+    if (col < ncols) tile[row][col] = in[(size_t)(kt * 2 + row) * size_n + ncol0 + col];
+  }
+  __syncthreads();
+
+  const int nt = t >> 7;        // n-tile inside the 128-column span
+  const int th = (t >> 2) & 31; // "thread" of the Marlin fragment
+  const int w = t & 3;
+  if (nt * 64 >= ncols) return;
+  const int r = 2 * (th & 3);
+  const int c = th >> 2;
+  const int n0 = nt * 64 + 16 * w + c;
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int kk = r + kDK[j];                 // row inside the k-tile
+    const int nn = n0 + ((j >> 1) & 1) * 8;
+    uint32_t src;
+    int nib;
+    if (HAS_PERM) {
+      src = tile[kk][nn];
+      nib = src_row[kk] & 7;
+    } else {
+      src = tile[kk >> 3][nn];
+      nib = kk & 7;
+    }
+    word |= ((src >> (4 * nib)) & 0xFu) << (4 * j);
+  }
+  out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
+}
+
+// AWQ source: word (k, cw), nibble t = q[k, 8*cw + {0,2,4,6,1,3,5,7}[t]]  =>  column 8*cw + j sits
+// in nibble {0,4,1,5,2,6,3,7}[j].
+__global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restrict__ in,
+                                                         uint32_t* __restrict__ out, int size_k,
+                                                         int size_n) {
+  __shared__ uint32_t tile[16][16];  // 16 rows x 16 words (128 columns)
+  const int t = threadIdx.x;
+  const int kt = blockIdx.y;
+  const int ncol0 = blockIdx.x * 128;
+  const int ncols = min(128, size_n - ncol0);
+  {
+    const int row = t >> 4, cw = t & 15;
+    if (cw * 8 < ncols) tile[row][cw] = in[(size_t)(kt * 16 + row) * (size_n >> 3) + (ncol0 >> 3) + cw];
+  }
+  __syncthreads();
+  const int nt = t >> 7;
+  const int th = (t >> 2) & 31;
+  const int w = t & 3;
+  if (nt * 64 >= ncols) return;
+  const int r = 2 * (th & 3);
+  const int c = th >> 2;
+  const int n0 = nt * 64 + 16 * w + c;
+  const int nib = ((c & 1) << 2) | (c >> 1);  // {0,4,1,5,2,6,3,7}[c]; n0 % 8 == c
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int kk = r + kDK[j];
+    const int nn = n0 + ((j >> 1) & 1) * 8;
+    const uint32_t src = tile[kk][nn >> 3];
+    word |= ((src >> (4 * nib)) & 0xFu) << (4 * j);
+  }
+  out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
+}
+
+// out[m, k] = a[m, perm[k]], 16-bit elements.
+__global__ __launch_bounds__(256) void permute_cols_kernel(const uint16_t* __restrict__ a,
+                                                           const int32_t* __restrict__ perm,
+                                                           uint16_t* __restrict__ out, int size_m,
+                                                           int size_k, int64_t lda) {
+  const int m = blockIdx.y;
+  for (int k = blockIdx.x * 256 + threadIdx.x; k < size_k; k += gridDim.x * 256)
+    out[(size_t)m * size_k + k] = a[(size_t)m * lda + perm[k]];
+}
+
+static int check_repack(int64_t size_k, int64_t size_n, int num_bits) {
+  W4A16_CHECK(size_k % 16 == 0, "size_k = %lld is not divisible by tile_k_size = 16", (long long)size_k);
+  W4A16_CHECK(size_n % 64 == 0, "size_n = %lld is not divisible by tile_n_size = 64", (long long)size_n);
+  W4A16_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = %d", num_bits);
+  if (num_bits == 8) return fail(W4A16_ENOTIMPL, "8-bit Marlin repack is not implemented in this build");
+  W4A16_CHECK(size_k / 16 <= 65535, "size_k = %lld too large", (long long)size_k);
+  return 0;
+}
+
+}  // namespace w4a16
+
+using namespace w4a16;
+
+extern "C" int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm, uint32_t* out,
+                                        int64_t size_k, int64_t size_n, int num_bits, void* stream) {
+  if (int rc = check_repack(size_k, size_n, num_bits)) return rc;
+  W4A16_CHECK(b_q_weight && out, "null weight pointer");
+  if (size_k == 0 || size_n == 0) return 0;
+  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
+  hipStream_t s = (hipStream_t)stream;
+  if (perm)
+    gptq_repack_kernel<true><<<grid, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n);
+  else
+    gptq_repack_kernel<false><<<grid, 256, 0, s>>>(b_q_weight, nullptr, out, (int)size_k, (int)size_n);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
+                                       int64_t size_n, int num_bits, void* stream) {
+  if (int rc = check_repack(size_k, size_n, num_bits)) return rc;
+  W4A16_CHECK(b_q_weight && out, "null weight pointer");
+  if (size_k == 0 || size_n == 0) return 0;
+  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
+  awq_repack_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k, (int)size_n);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_permute_cols(const void* a, const int32_t* perm, void* out, int64_t size_m,
+                                  int64_t size_k, int64_t lda, void* stream) {
+  W4A16_CHECK(a && perm && out, "null pointer");
+  W4A16_CHECK(size_m <= 65535 * 1024LL, "size_m too large");
+  if (size_m == 0 || size_k == 0) return 0;
+  // grid.y is limited to 65535: walk M in slabs
+  for (int64_t m0 = 0; m0 < size_m; m0 += 65535) {
+    const int rows = (int)((size_m - m0) < 65535 ? (size_m - m0) : 65535);
+    dim3 grid((unsigned)((size_k + 255) / 256 < 64 ? (size_k + 255) / 256 : 64), (unsigned)rows);
+    permute_cols_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)a + m0 * lda, perm, (uint16_t*)out + m0 * size_k, rows, (int)size_k, lda);
+  }
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}

@@ -1,0 +1,179 @@
+"""Host-side helpers of the Marlin linear path, mirroring the reference's
+vllm/model_executor/layers/quantization/utils/marlin_utils.py (names, arguments and results),
+restricted to what the 4-bit GPTQ / AWQ path needs.  All tensor work runs on the tensor's device.
+"""
+import os
+
+import torch
+
+from . import _custom_ops as ops
+from .quant_utils import pack_cols, unpack_cols
+from .scalar_type import ScalarType, scalar_types
+
+GPTQ_MARLIN_TILE = 16
+GPTQ_MARLIN_MIN_THREAD_N = 64
+GPTQ_MARLIN_MIN_THREAD_K = 128
+GPTQ_MARLIN_MAX_PARALLEL = 16
+
+MARLIN_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
+USE_FP32_REDUCE_DEFAULT = True
+
+_INTERLEAVE_4BIT = (0, 2, 4, 6, 1, 3, 5, 7)
+
+
+def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True,
+                                       device_capability: int | None = None) -> list[ScalarType]:
+    """marlin_utils.py:35-78, narrowed to the types this library implements (4-bit)."""
+    if has_zp is None:
+        return (query_marlin_supported_quant_types(False, include_fp_type, device_capability) +
+                query_marlin_supported_quant_types(True, include_fp_type, device_capability))
+    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8]
+
+
+def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,
+                                input_size: int, group_size: int) -> tuple[bool, str | None]:
+    """marlin_utils.py:126-175 (same gates, same messages)."""
+    try:
+        verify_marlin_supports_shape(output_size_per_partition, input_size_per_partition, input_size, group_size)
+    except ValueError as e:
+        return False, str(e)
+    return True, None
+
+
+def verify_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,
+                                 input_size: int, group_size: int) -> None:
+    if output_size_per_partition % GPTQ_MARLIN_MIN_THREAD_N != 0:
+        raise ValueError(f"Weight output_size_per_partition = {output_size_per_partition} is not divisible by "
+                         f" min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}. Consider reducing tensor_parallel_size or "
+                         "running with --quantization gptq.")
+    if input_size_per_partition % GPTQ_MARLIN_MIN_THREAD_K != 0:
+        raise ValueError(f"Weight input_size_per_partition = {input_size_per_partition} is not divisible by "
+                         f"min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}. Consider reducing tensor_parallel_size or "
+                         "running with --quantization gptq.")
+    if group_size < input_size and input_size_per_partition % group_size != 0:
+        raise ValueError(f"Weight input_size_per_partition = {input_size_per_partition} is not divisible by "
+                         f"group_size = {group_size}. Consider reducing tensor_parallel_size or running with "
+                         "--quantization gptq.")
+
+
+def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1) -> torch.Tensor:
+    """int32 zeros, one counter per compute unit (x max_blocks_per_sm); marlin_utils.py:237-245.
+    The GEMM keeps the all-zero-on-exit invariant, so one workspace serves any number of calls."""
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    return torch.zeros(cus * max_blocks_per_sm, dtype=torch.int, device=device, requires_grad=False)
+
+
+def marlin_is_k_full(act_order: bool, is_row_parallel: bool) -> bool:
+    return (not act_order) or (act_order and not is_row_parallel)
+
+
+def marlin_repeat_scales_on_all_ranks(act_order: bool, group_size: int, is_row_parallel: bool) -> bool:
+    return act_order or (group_size == -1 and is_row_parallel)
+
+
+def marlin_make_empty_g_idx(device: torch.device) -> torch.Tensor:
+    return torch.nn.Parameter(torch.empty(0, dtype=torch.int, device=device), requires_grad=False)
+
+
+def marlin_make_empty_zp(device: torch.device) -> torch.Tensor:
+    return torch.nn.Parameter(torch.empty(0, dtype=torch.int, device=device), requires_grad=False)
+
+
+def marlin_sort_g_idx(g_idx: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    g_idx_sort_indices = torch.argsort(g_idx).to(torch.int)
+    return g_idx[g_idx_sort_indices.long()], g_idx_sort_indices
+
+
+def get_scale_perms() -> tuple[list[int], list[int]]:
+    scale_perm = [i + 8 * j for i in range(8) for j in range(8)]
+    scale_perm_single = [2 * i + j for i in range(4) for j in (0, 1, 8, 9, 16, 17, 24, 25)]
+    return scale_perm, scale_perm_single
+
+
+def marlin_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int) -> torch.Tensor:
+    scale_perm, scale_perm_single = get_scale_perms()
+    perm = scale_perm if (group_size < size_k and group_size != -1) else scale_perm_single
+    idx = torch.tensor(perm, device=s.device)
+    return s.reshape((-1, len(perm)))[:, idx].reshape((-1, size_n)).contiguous()
+
+
+def marlin_permute_bias(s: torch.Tensor) -> torch.Tensor:
+    _, scale_perm_single = get_scale_perms()
+    idx = torch.tensor(scale_perm_single, device=s.device)
+    return s.reshape((-1, len(scale_perm_single)))[:, idx].reshape(s.shape).contiguous()
+
+
+def marlin_moe_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int) -> torch.Tensor:
+    out = torch.empty_like(s)
+    for e in range(s.shape[0]):
+        out[e] = marlin_permute_scales(s[e], size_k, size_n, group_size)
+    return out
+
+
+def marlin_zero_points(zp: torch.Tensor, size_k: int, size_n: int, num_bits: int) -> torch.Tensor:
+    """Unpacked zero points [size_k(=groups), size_n] -> Marlin-packed int32 [groups, size_n/8]
+    (marlin_utils.py:326-346)."""
+    assert num_bits == 4, "only 4-bit zero points are implemented"
+    scale_perm, _ = get_scale_perms()
+    zp = zp.reshape((-1, len(scale_perm)))[:, torch.tensor(scale_perm, device=zp.device)]
+    inter = torch.tensor(_INTERLEAVE_4BIT, device=zp.device)
+    zp = zp.reshape((-1, len(_INTERLEAVE_4BIT)))[:, inter].reshape((-1, size_n)).contiguous()
+    return pack_cols(zp, num_bits, size_k, size_n)
+
+
+def awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int) -> torch.Tensor:
+    """AWQ-packed zero points -> Marlin-packed (marlin_utils.py:349-370)."""
+    assert num_bits == 4, "only 4-bit zero points are implemented"
+    q_zp = unpack_cols(q_zp_packed, num_bits, size_k, size_n)
+    undo = torch.argsort(torch.tensor(_INTERLEAVE_4BIT, device=q_zp.device))
+    q_zp = q_zp.reshape((-1, len(_INTERLEAVE_4BIT)))[:, undo].reshape((-1, size_n)).contiguous()
+    return marlin_zero_points(q_zp, size_k, size_n, num_bits)
+
+
+def moe_awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int):
+    out = torch.empty_like(q_zp_packed)
+    for e in range(q_zp_packed.shape[0]):
+        out[e] = awq_to_marlin_zero_points(q_zp_packed[e], size_k, size_n, num_bits)
+    return out
+
+
+def should_use_atomic_add_reduce(m: int, n: int, k: int, device: torch.device, dtype: torch.dtype) -> bool:
+    """marlin_utils.py:412-432.  The flag is forwarded for interface parity; the gfx950 kernels
+    always reduce split-K partials in a fixed order in fp32."""
+    if n >= 2048 or k < 2048 or device.type != "cuda":
+        return False
+    return os.environ.get("VLLM_MARLIN_USE_ATOMIC_ADD", "0") == "1"
+
+
+def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                             weight_zp: torch.Tensor, g_idx: torch.Tensor, g_idx_sort_indices: torch.Tensor,
+                             workspace: torch.Tensor, wtype: ScalarType, output_size_per_partition: int,
+                             input_size_per_partition: int, is_k_full: bool, bias: torch.Tensor | None = None,
+                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    reshaped_x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (output_size_per_partition,)
+    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
+                                                  reshaped_x.size(1), input.device, input.dtype)
+    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, weight_zp, g_idx,
+                                  g_idx_sort_indices, workspace, wtype, size_m=reshaped_x.shape[0],
+                                  size_n=output_size_per_partition, size_k=input_size_per_partition,
+                                  is_k_full=is_k_full, use_atomic_add=use_atomic_add,
+                                  use_fp32_reduce=use_fp32_reduce, is_zp_float=False)
+    return output.reshape(out_shape)
+
+
+def apply_awq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                            weight_zp: torch.Tensor, g_idx: torch.Tensor, g_idx_sort_indices: torch.Tensor,
+                            workspace: torch.Tensor, quant_type: ScalarType, output_size_per_partition: int,
+                            input_size_per_partition: int, bias: torch.Tensor | None = None,
+                            use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    reshaped_x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (output_size_per_partition,)
+    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
+                                                  reshaped_x.size(1), input.device, input.dtype)
+    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, weight_zp, g_idx,
+                                  g_idx_sort_indices, workspace, quant_type, size_m=reshaped_x.shape[0],
+                                  size_n=output_size_per_partition, size_k=input_size_per_partition,
+                                  use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,
+                                  is_zp_float=False)
+    return output.reshape(out_shape)
