@@ -1,0 +1,307 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A16 Marlin-surface GEMM on one MI355X.
+
+Default workload (`config.workload`): the four Llama-3-8B decode linears
+(K,N) = (4096,6144) qkv, (4096,4096) o, (4096,28672) gate_up, (14336,4096) down at M = 16,
+GPTQ uint4b8, group 128, fp16, no act-order.  One "step" = those four GEMMs, each on a weight
+copy that has not been touched for >= 512 MB of other traffic (cold for L2 and the 256 MB
+Infinity Cache), inputs resident in HBM, replayed from a HIP graph so host launch cost is not in
+the timed region.  `value` = algorithmic bytes of the step / time = GB/s.
+
+Also printed in the same JSON line:
+  roofline      algorithmic bytes per launch / average launch duration (HIP events on the launch
+                stream) against the 8 TB/s HBM peak, for the decode kernel
+  cpu_baseline  the oracle's dequantize + torch.matmul path on the host cores, bounded sample
+  detail        per-shape µs / GB/s / TFLOP/s / roofline fractions (decode M in {1,4,16,64,256},
+                prefill M = 4096 bf16 AWQ; the latter against the 2.5 PFLOP/s dense MFMA peak)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0
+LAYERS = {"qkv": (4096, 6144), "o": (4096, 4096), "gate_up": (4096, 28672), "down": (14336, 4096)}
+GROUP = 128
+
+
+def algorithmic_bytes(m, k, n, zp=False, act_order=False):
+    b = k * n // 2 + (k // GROUP) * n * 2 + m * k * 2 + m * n * 2
+    if zp:
+        b += (k // GROUP) * n // 2
+    if act_order:
+        b += 2 * k * 4
+    return b
+
+
+# ------------------------------------------------------------------ synthetic layers (on the GPU)
+def _pack_rows_gpu(q):  # [K, N] int -> GPTQ int32 [K/8, N]
+    k, n = q.shape
+    f = q.to(torch.int64).reshape(k // 8, 8, n)
+    sh = (torch.arange(8, device=q.device, dtype=torch.int64) * 4).view(1, 8, 1)
+    w = (f << sh).sum(dim=1)
+    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32).contiguous()
+
+
+def _pack_cols_awq_gpu(q):  # [K, N] int -> AWQ int32 [K, N/8]
+    k, n = q.shape
+    order = torch.tensor([0, 2, 4, 6, 1, 3, 5, 7], device=q.device)
+    f = q.to(torch.int64).reshape(k, n // 8, 8)[:, :, order]
+    sh = (torch.arange(8, device=q.device, dtype=torch.int64) * 4).view(1, 1, 8)
+    w = (f << sh).sum(dim=2)
+    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32).contiguous()
+
+
+def make_gptq_layer(ops, k, n, dtype, dev, seed):
+    """N(0, 0.02) weights, symmetric uint4b8 RTN, s = absmax/7 per (group, column)."""
+    from vllm_amd.marlin_utils import marlin_permute_scales
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    w = (torch.randn(k, n, generator=g) * 0.02).to(dtype).to(dev)
+    wg = w.float().reshape(k // GROUP, GROUP, n)
+    s = (wg.abs().amax(dim=1, keepdim=True) / 7).clamp(min=1e-5).to(dtype)
+    q = torch.clamp(torch.round(wg / s.float()), -8, 7).to(torch.int32)
+    w_deq = (q.to(dtype) * s).reshape(k, n)
+    packed = _pack_rows_gpu((q + 8).reshape(k, n))
+    mq = ops.gptq_marlin_repack(packed, torch.empty(0, dtype=torch.int32, device=dev), k, n, 4)
+    ms = marlin_permute_scales(s.reshape(k // GROUP, n), k, n, GROUP)
+    return {"k": k, "n": n, "q": mq, "s": ms, "zp": torch.empty(0, dtype=torch.int32, device=dev), "w_deq": w_deq,
+            "packed": packed, "scales": s.reshape(k // GROUP, n)}
+
+
+def make_awq_layer(ops, k, n, dtype, dev, seed):
+    """N(0, 0.02) weights, asymmetric uint4 RTN from per-group min/max, uint4 zero points."""
+    from vllm_amd.marlin_utils import awq_to_marlin_zero_points, marlin_permute_scales
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    w = (torch.randn(k, n, generator=g) * 0.02).to(dtype).to(dev)
+    wg = w.float().reshape(k // GROUP, GROUP, n)
+    hi, lo = wg.amax(dim=1, keepdim=True), wg.amin(dim=1, keepdim=True)
+    s = ((hi - lo) / 15).clamp(min=1e-5).to(dtype)
+    z = torch.clamp(torch.round(-lo / s.float()), 0, 15).to(torch.int32)
+    q = torch.clamp(torch.round(wg / s.float()).to(torch.int32) + z, 0, 15)
+    w_deq = ((q - z).to(dtype) * s).reshape(k, n)
+    mq = ops.awq_marlin_repack(_pack_cols_awq_gpu(q.reshape(k, n)), k, n, 4)
+    ms = marlin_permute_scales(s.reshape(k // GROUP, n), k, n, GROUP)
+    mz = awq_to_marlin_zero_points(_pack_cols_awq_gpu(z.reshape(k // GROUP, n)), k // GROUP, n, 4)
+    return {"k": k, "n": n, "q": mq, "s": ms, "zp": mz, "w_deq": w_deq}
+
+
+def clone_weights(layer, seed):
+    """A distinct copy of the streamed operands (random nibbles, same scales): only used to rotate
+    buffers so that no launch finds its weights in a cache."""
+    g = torch.Generator(device=layer["q"].device).manual_seed(seed)
+    q = torch.randint(-2**31, 2**31 - 1, layer["q"].shape, generator=g, device=layer["q"].device, dtype=torch.int32)
+    return {**layer, "q": q, "s": layer["s"].clone(), "zp": layer["zp"].clone(), "w_deq": None}
+
+
+def gemm(ops, wtype, a, layer, workspace):
+    e = torch.empty(0, dtype=torch.int32, device=a.device)
+    return ops.gptq_marlin_gemm(a, None, layer["q"], None, layer["s"], None, layer["zp"], e, e, workspace, wtype,
+                                a.shape[0], layer["n"], layer["k"], True, False, True, False)
+
+
+def time_graph(fn_list, reps, warmup):
+    """Capture `fn_list` (a list of zero-arg launch closures) into one HIP graph, replay it `warmup`
+    times untimed and `reps` times between two events on the launch stream; returns seconds/replay."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for f in fn_list:  # eager warm-up (module load, allocator)
+            f()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for f in fn_list:
+                f()
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record(stream)
+        for _ in range(reps):
+            graph.replay()
+        t1.record(stream)
+        torch.cuda.synchronize()
+    return t0.elapsed_time(t1) * 1e-3 / reps
+
+
+def copies_needed(weight_bytes):
+    return max(2, -(-512 * 2**20 // weight_bytes) + 1)
+
+
+def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=40, zp=False):
+    """Cold (rotating weight copies) time of one shape; returns dict."""
+    base = layer_fn(k, n, dtype, dev, 1)
+    wbytes = base["q"].numel() * 4
+    ncopy = min(copies_needed(wbytes), 64)
+    copies = [base] + [clone_weights(base, 100 + i) for i in range(ncopy - 1)]
+    g = torch.Generator(device="cpu").manual_seed(2)
+    a = torch.randn(m, k, generator=g).to(dtype).to(dev)
+    out = gemm(ops, wtype, a, base, workspace)
+    ref = a.float() @ base["w_deq"].float()
+    err = float((out.float() - ref).abs().max() / ref.abs().max())
+    fns = [(lambda c=copies[i % ncopy]: gemm(ops, wtype, a, c, workspace)) for i in range(max(launches, ncopy))]
+    sec = time_graph(fns, reps=3, warmup=1) / len(fns)
+    warm = time_graph([lambda: gemm(ops, wtype, a, base, workspace)] * 20, reps=3, warmup=1) / 20
+    by, fl = algorithmic_bytes(m, k, n, zp=zp), 2.0 * m * n * k
+    del copies
+    torch.cuda.empty_cache()
+    return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_warm": warm * 1e6, "GBps": by / sec / 1e9,
+            "TFLOPs": fl / sec / 1e12, "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS,
+            "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS, "max_rel_err": err}
+
+
+def cpu_baseline(m, budget_s=25.0):
+    """The oracle's CPU path (unpack GPTQ nibbles, (q-8)*s group-broadcast, torch.matmul in fp32) on the
+    host cores, for as many of the four layers at M=`m` as fit the time budget (smallest first)."""
+    from oracle import gemm_ref as gr
+    from oracle import quant_utils as qu
+    torch.manual_seed(0)
+    done, t_total, b_total = [], 0.0, 0
+    for name, (k, n) in sorted(LAYERS.items(), key=lambda kv: kv[1][0] * kv[1][1]):
+        if t_total > budget_s * 0.5 and done:
+            break
+        q = torch.randint(0, 16, (k, n), dtype=torch.int32)
+        packed = qu.gptq_pack(q)
+        s = (torch.rand(k // GROUP, n) * 0.01 + 0.005).half()
+        a = torch.randn(m, k).half()
+        del q
+        t0 = time.perf_counter()
+        w = gr.dequant_checkpoint(packed, s, None, None, "gptq", torch.float16)
+        out = gr.gemm_ref(a, w)
+        dt = time.perf_counter() - t0
+        del w, out
+        done.append(name)
+        t_total += dt
+        b_total += algorithmic_bytes(m, k, n)
+    return {"value": b_total / t_total / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"dequantize+matmul of layers {done} at M={m}, one pass each, {t_total:.1f} s",
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--m", type=int, default=16, help="decode batch of the headline workload")
+    ap.add_argument("--no-detail", action="store_true", help="skip the per-shape table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--table", type=str, default="", help="also write the detail table to this JSON file")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.scalar_type import scalar_types
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    workspace = marlin_make_workspace_new(dev)
+    m = args.m
+
+    # ---- headline: one step = the four decode GEMMs, weights rotated over `nsets` full sets
+    step_wbytes = sum(k * n // 2 for k, n in LAYERS.values())
+    nsets = copies_needed(step_wbytes)
+    base = {name: make_gptq_layer(ops, k, n, torch.float16, dev, 10 + i) for i, (name, (k, n)) in enumerate(LAYERS.items())}
+    sets = [base] + [{name: clone_weights(l, 1000 * s + i) for i, (name, l) in enumerate(base.items())}
+                     for s in range(1, nsets)]
+    acts = {name: torch.randn(m, k, generator=torch.Generator().manual_seed(3)).half().to(dev)
+            for name, (k, n) in LAYERS.items()}
+    # correctness guard of the timed path (dequantised fp32 matmul on the GPU)
+    errs = {}
+    for name, l in base.items():
+        out = gemm(ops, scalar_types.uint4b8, acts[name], l, workspace)
+        ref = acts[name].float() @ l["w_deq"].float()
+        errs[name] = float((out.float() - ref).abs().max() / ref.abs().max())
+    assert max(errs.values()) < 2e-2, errs
+
+    def step(i):
+        s = sets[i % nsets]
+        for name in LAYERS:
+            gemm(ops, scalar_types.uint4b8, acts[name], s[name], workspace)
+
+    steps_per_graph = nsets
+    fns = [(lambda i=i: step(i)) for i in range(steps_per_graph)]
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for f in fns:
+            f()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for f in fns:
+                f()
+        done = 0
+        while done < args.warmup:
+            graph.replay()
+            done += steps_per_graph
+        torch.cuda.synchronize()
+        replays = -(-args.steps // steps_per_graph)
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record(stream)
+        for _ in range(replays):
+            graph.replay()
+        t1.record(stream)
+        torch.cuda.synchronize()
+    timed_steps = replays * steps_per_graph
+    sec_per_step = t0.elapsed_time(t1) * 1e-3 / timed_steps
+    step_bytes = sum(algorithmic_bytes(m, k, n) for k, n in LAYERS.values())
+    value = step_bytes / sec_per_step / 1e9
+    launches = 4 * timed_steps
+    avg_launch_s = sec_per_step / 4
+
+    result = {
+        "metric": "W4A16 GEMM algorithmic HBM GB/s, Llama-3-8B decode linears (qkv,o,gate_up,down)",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": timed_steps, "warmup": args.warmup,
+        "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"llama3-8b decode linears M={m}, GPTQ uint4b8 g128 fp16, no act-order, cold weights",
+                   "shapes_KN": list(LAYERS.values()), "M": m, "weight_sets_rotated": nsets,
+                   "timing": "HIP graph replay between two events on the launch stream"},
+        "roofline": {"bound": "hbm", "achieved": step_bytes / 4 / avg_launch_s / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": step_bytes / 4 / avg_launch_s / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "skinny_kernel<f16, MB=1, no-zp, grouped>", "launches": launches,
+                     "avg_launch_us": avg_launch_s * 1e6, "algorithmic_bytes_per_launch": step_bytes / 4},
+        "us_per_gemm_avg": avg_launch_s * 1e6,
+        "max_rel_err_vs_fp32": errs,
+    }
+    del sets, base
+    torch.cuda.empty_cache()
+
+    if not args.no_detail:
+        detail = {"decode_fp16_gptq": {}, "prefill_bf16_awq": {}}
+        for name, (k, n) in LAYERS.items():
+            for mm in (1, 4, 16, 64, 256):
+                r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_layer(ops, *a), mm, k, n,
+                                torch.float16, dev, workspace)
+                detail["decode_fp16_gptq"][f"{name}_M{mm}"] = r
+                print(f"[detail] {name} M={mm}: {r['us']:.2f} us cold ({r['us_warm']:.2f} warm), "
+                      f"{r['GBps']:.0f} GB/s = {100 * r['hbm_frac']:.1f}% HBM, {r['TFLOPs']:.1f} TFLOP/s",
+                      file=sys.stderr, flush=True)
+        for name, (k, n) in LAYERS.items():
+            r = bench_shape(ops, scalar_types.uint4, lambda *a: make_awq_layer(ops, *a), 4096, k, n, torch.bfloat16,
+                            dev, workspace, launches=8, zp=True)
+            detail["prefill_bf16_awq"][f"{name}_M4096"] = r
+            print(f"[detail] {name} M=4096 bf16 awq: {r['us']:.1f} us, {r['TFLOPs']:.1f} TFLOP/s = "
+                  f"{100 * r['mfma_frac']:.1f}% MFMA peak", file=sys.stderr, flush=True)
+        result["detail"] = detail
+        if args.table:
+            with open(args.table, "w") as f:
+                json.dump(detail, f, indent=1)
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(m)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

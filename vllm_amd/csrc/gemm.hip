@@ -86,20 +86,21 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   pl.tiles = (int)tiles;
   pl.total_ksteps = (int)(a->size_k / 32);
 
+  // One workgroup (8 wavefronts) per compute unit: split K until the grid covers the chip, keeping at
+  // least one k-step per wavefront.  Splitting needs one counter per tile in the caller's workspace.
   static const int forced_splits = env_int("W4A16_SPLITS", 0);
-  static const int target_mult = env_int("W4A16_TARGET_WG_PER_CU", 2);
+  static const int target_mult = env_int("W4A16_TARGET_WG_PER_CU", 1);
   const int target = num_cus() * target_mult;
   int splits = 1;
   if (pl.tiles > 0 && pl.tiles < target && a->workspace && pl.tiles <= a->workspace_len) {
-    splits = (int)ceil_div(target, pl.tiles);
-    const int max_splits = pl.total_ksteps / 4 > 0 ? pl.total_ksteps / 4 : 1;
+    splits = (target + pl.tiles / 2) / pl.tiles;
+    const int max_splits = pl.total_ksteps / 8 > 0 ? pl.total_ksteps / 8 : 1;
+    if (forced_splits > 0) splits = forced_splits;
     if (splits > max_splits) splits = max_splits;
-    if (forced_splits > 0) splits = forced_splits < max_splits ? forced_splits : max_splits;
+    if (splits < 1) splits = 1;
   }
-  int kps = (int)ceil_div(pl.total_ksteps, splits);
-  kps = (kps + 3) & ~3;
-  pl.kps = kps;
-  pl.splits = (int)ceil_div(pl.total_ksteps, kps);
+  pl.kps = (int)ceil_div(pl.total_ksteps, splits);
+  pl.splits = (int)ceil_div(pl.total_ksteps, pl.kps);
   pl.xcd_map = (pl.splits > 1 && pl.tiles % 8 == 0) ? 1 : 0;
   pl.ctmp_bytes = pl.splits > 1 ? (int64_t)pl.tiles * pl.splits * pl.bm * 128 * 4 : 0;
   return 0;

@@ -110,7 +110,10 @@ template <int DT, bool UNIT_SCALE>
 __device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const ColConst<DT>& cc, u32x4& o0,
                                              u32x4& o1) {
   if constexpr (DT == DT_F16) {
-    const uint32_t MLO = 0x000f000fu, MHI = 0x00f000f0u, EX = 0x64006400u;
+    const uint32_t MLO = 0x000f000fu, MHI = 0x00f000f0u;
+    // keep the exponent pattern in a VGPR so that (x & mask) | EX is one v_and_or_b32
+    uint32_t EX = 0x64006400u;
+    asm("" : "+v"(EX));
     const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
     const f16x2 s = as_h2(cc.s), zl = as_h2(cc.zl), zh = as_h2(cc.zh);
     const f16x2 s0 = {s.x, s.x}, s1 = {s.y, s.y};
