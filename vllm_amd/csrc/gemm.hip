@@ -80,29 +80,68 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.bm = 16 * pl.mb;
     pl.mtiles = (int)ceil_div(a->size_m, pl.bm);
   }
-  pl.ncp = (int)ceil_div(a->size_n, 128);
-  const int64_t tiles = (int64_t)pl.mtiles * pl.ncp;
-  W4A16_CHECK(tiles < (1LL << 31) / 64, "too many tiles");
-  pl.tiles = (int)tiles;
   pl.total_ksteps = (int)(a->size_k / 32);
-
-  // One workgroup (8 wavefronts) per compute unit: split K until the grid covers the chip, keeping at
-  // least one k-step per wavefront.  Splitting needs one counter per tile in the caller's workspace.
+  const int cus = num_cus();
   static const int forced_splits = env_int("W4A16_SPLITS", 0);
-  static const int target_mult = env_int("W4A16_TARGET_WG_PER_CU", 1);
-  const int target = num_cus() * target_mult;
-  int splits = 1;
-  if (pl.tiles > 0 && pl.tiles < target && a->workspace && pl.tiles <= a->workspace_len) {
-    splits = (target + pl.tiles / 2) / pl.tiles;
-    const int max_splits = pl.total_ksteps / 8 > 0 ? pl.total_ksteps / 8 : 1;
-    if (forced_splits > 0) splits = forced_splits;
-    if (splits > max_splits) splits = max_splits;
-    if (splits < 1) splits = 1;
+  static const int forced_tn = env_int("W4A16_TN", 0);
+  static const int forced_kind = env_int("W4A16_KIND", -1);
+
+  // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
+  const bool decode_ok = pl.mb == 1 && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
+                         (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
+
+  // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these
+  // kernels: one 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~21 GB/s on a 64-column
+  // strip (instruction-issue bound), the whole chip ~4.7 TB/s; summing K-splits across workgroups adds
+  // ~3 us of dependent device-scope round trips.  Only one such workgroup fits a compute unit, so a grid
+  // larger than the number of compute units runs in rounds.  Each split needs >= 1 stage per wavefront and
+  // one workspace counter per tile.
+  struct Cand { int kind, tn, splits; double t; };
+  Cand best{0, 128, 1, 1e30};
+  const int n_tn = decode_ok ? 2 : 1;
+  for (int ti = 0; ti < n_tn; ++ti) {
+    const int tn = ti == 0 ? 128 : 64;
+    if (forced_tn && tn != forced_tn && decode_ok) continue;
+    const int64_t ncol_tiles = ceil_div(a->size_n, tn);
+    const int64_t tiles = (int64_t)pl.mtiles * ncol_tiles;
+    if (tiles <= 0 || tiles >= (1LL << 31) / 64) continue;
+    const double bytes = (double)tiles * a->size_k * tn / 2.0;
+    const double wg_rate = (tn == 64 ? 21e3 : 33e3) / (pl.mb > 1 ? 1.5 : 1.0);  // bytes per us
+    const double chip_rate = 4.7e6;
+    const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
+    const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
+    for (int sp = 1; sp <= 16; ++sp) {
+      if (sp > max_splits) break;
+      if (sp > 1 && (!a->workspace || tiles > a->workspace_len)) break;
+      if (forced_splits > 0 && sp != (forced_splits < max_splits ? forced_splits : max_splits)) continue;
+      const int64_t wgs = tiles * sp;
+      if (sp > 1 && wgs > cus) break;
+      const int64_t rounds = ceil_div(wgs, cus);
+      double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
+      if (rate > chip_rate) rate = chip_rate;
+      const double t = bytes / rate + (sp > 1 ? 2.8 + 0.05 * sp : 0.0);
+      if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, t};
+    }
   }
-  pl.kps = (int)ceil_div(pl.total_ksteps, splits);
-  pl.splits = (int)ceil_div(pl.total_ksteps, pl.kps);
+  W4A16_CHECK(best.t < 1e30, "no launch shape for this problem (too many tiles)");
+  pl.kind = best.kind;
+  pl.tn = best.tn;
+  pl.ncp = (int)ceil_div(a->size_n, pl.tn);
+  pl.tiles = pl.mtiles * pl.ncp;
+  {
+    const int align = pl.kind == 1 ? 2 : 1;  // decode stages are two k-steps
+    int kps = (int)ceil_div(pl.total_ksteps, best.splits);
+    kps = (kps + align - 1) / align * align;
+    pl.kps = kps;
+    pl.splits = (int)ceil_div(pl.total_ksteps, kps);
+  }
+  static const int debug = env_int("W4A16_DEBUG", 0);
+  if (debug)
+    fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=%d tn=%d mb=%d tiles=%d splits=%d kps=%d model_us=%.2f\n",
+            (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, pl.kind, pl.tn, pl.mb, pl.tiles,
+            pl.splits, pl.kps, best.t);
   pl.xcd_map = (pl.splits > 1 && pl.tiles % 8 == 0) ? 1 : 0;
-  pl.ctmp_bytes = pl.splits > 1 ? (int64_t)pl.tiles * pl.splits * pl.bm * 128 * 4 : 0;
+  pl.ctmp_bytes = pl.splits > 1 ? (int64_t)pl.tiles * pl.splits * pl.bm * pl.tn * 4 : 0;
   return 0;
 }
 
@@ -125,5 +164,5 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
   if (int rc = make_plan(args, pl)) return rc;
   if (pl.mtiles == 0) return 0;
   if (pl.ctmp_bytes > 0) W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed", (long long)pl.ctmp_bytes);
-  return launch_skinny(args, pl, (hipStream_t)stream);
+  return pl.kind == 1 ? launch_decode(args, pl, (hipStream_t)stream) : launch_skinny(args, pl, (hipStream_t)stream);
 }

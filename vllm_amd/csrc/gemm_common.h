@@ -152,6 +152,27 @@ __device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const Col
   }
 }
 
+// "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
+// of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
+// high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the
+// caller compensates by scaling the matching activations by 1/16.  No subtract, no scale: both are
+// applied to the fp32 accumulator once per quantization group.
+template <int DT, bool HI_TRICK>
+__device__ __forceinline__ void raw_pair(uint32_t xa, uint32_t xb, u32x4& o0, u32x4& o1) {
+  const uint32_t M = 0x000f000fu;
+  uint32_t E = (DT == DT_F16) ? 0x64006400u : 0x43004300u;
+  asm("" : "+v"(E));  // keep in a VGPR: (x & mask) | E becomes one v_and_or_b32
+  if constexpr (HI_TRICK) {
+    const uint32_t MH = 0x00f000f0u;
+    const uint32_t ya = xa >> 8, yb = xb >> 8;
+    o0 = u32x4{(xa & M) | E, (xa & MH) | E, (xb & M) | E, (xb & MH) | E};
+    o1 = u32x4{(ya & M) | E, (ya & MH) | E, (yb & M) | E, (yb & MH) | E};
+  } else {
+    o0 = u32x4{(xa & M) | E, ((xa >> 4) & M) | E, (xb & M) | E, ((xb >> 4) & M) | E};
+    o1 = u32x4{((xa >> 8) & M) | E, ((xa >> 12) & M) | E, ((xb >> 8) & M) | E, ((xb >> 12) & M) | E};
+  }
+}
+
 // Position of real column `cl` (0..31 inside its 32-column chunk) in a tensor permuted with the
 // reference's "single" permutation (marlin_utils.py:278-286, used for channel-wise scales and bias).
 __device__ __forceinline__ int single_perm_pos(int cl) {

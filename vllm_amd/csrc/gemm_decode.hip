@@ -1,0 +1,448 @@
+// W4A16 decode GEMM for gfx950 (M-tiles of 16 rows): C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias).
+//
+// Specialisation of the skinny kernel for the weight-streaming regime, where the kernel is bound by HBM
+// and by fixed latencies rather than by the matrix cores.  Same operand layouts and the same workgroup
+// decomposition (tile x split, 8 wavefronts cutting the split's K range into contiguous parts, LDS sum,
+// ordered cross-workgroup sum), with these differences:
+//   * tile width TN = 128 columns (a column pair, 128-bit loads) or 64 columns (one n-tile, 64-bit loads);
+//     narrow tiles give twice as many workgroups, so small-N layers can cover enough compute units without
+//     splitting K across workgroups (a cross-workgroup sum costs ~4 us of dependent device-scope round trips).
+//   * a pipeline stage is two k-steps (64 K rows): 4 weight loads, 2 activation loads that read 128
+//     contiguous bytes per row (full cache lines), one scale load, one zero-point load.
+//   * "fold" arithmetic: nibbles are only OR-ed into the mantissa of a magic exponent (fp16: 1024+q or, for
+//     the high nibbles, 1024+16q against activations pre-scaled by 1/16; bf16: 128+q) and fed to the MFMA as
+//     they are; one extra MFMA per k-step against a constant operand accumulates the bias term
+//     sum_k a_k * (E+8)  [or sum_k a_k when zero points vary per column].  Once per quantization group the fp32
+//     partial is folded:  acc += s * (tmp - (E+z) * rs).  Exact integer dequantisation happens in fp32, the
+//     scale is applied once per group in fp32; a one-hot activation row still reproduces half(q-z)*half(s)
+//     rounded once, bit for bit.  ~45 VALU instructions per k-step instead of ~135.
+// Requirements (checked on the host, which otherwise falls back to the skinny kernel): K % 64 == 0,
+// group size a multiple of 64 (or channel-wise), no per-row g_idx lookup.
+#include "gemm_kernels.h"
+
+namespace w4a16 {
+
+constexpr int DNW = 8;  // wavefronts per workgroup
+constexpr int DD = 3;   // stages (of two k-steps) in flight per wavefront
+
+template <int TN>
+struct DecodeCfg {
+  static constexpr int RS = (TN == 128) ? RED_RS : 84;  // reduction slab row stride (floats), 4 mod 16
+  static constexpr int SMEM = DNW * 16 * RS * 4;
+};
+
+template <int DT, bool ZP, bool CHANNEL, bool PERM, int TN>
+__global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
+  constexpr int W = TN / 32;  // Marlin words per lane and k-tile: 4 (128-bit load) or 2 (64-bit load)
+  constexpr bool HI_TRICK = (DT == DT_F16) && !ZP;
+  constexpr int RS = DecodeCfg<TN>::RS;
+  using bvec = uint32_t __attribute__((ext_vector_type(W)));
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int s_crow[16];
+  __shared__ int s_last;
+
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // weight-side roles: c = column inside an 8-column block, h = which half of the tile's columns, g = K group
+  const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
+
+  int tile, split;
+  {
+    const int b = blockIdx.x;
+    if (p.xcd_map) {
+      const int idx = b >> 3;
+      tile = (idx / p.splits) * 8 + (b & 7);
+      split = idx % p.splits;
+    } else {
+      tile = b / p.splits;
+      split = b % p.splits;
+    }
+  }
+  const int ct = tile % p.ncp, mt = tile / p.ncp;  // column tile, m-tile
+
+  const uint32_t* Bq = p.B;
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint32_t* Zp = p.Z;
+  const int32_t* perm = p.perm;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  if (p.moe) {
+    if (mt * p.moe_bs >= *p.ntpp) return;
+    const int e = p.expert_ids[mt];
+    if (e < 0) return;
+    Bq += e * p.b_estride;
+    Sc += e * p.s_estride;
+    if (ZP) Zp += e * p.z_estride;
+    if (PERM) perm += e * p.k_estride;
+    if (bias) bias += e * p.n_estride;
+  }
+
+  auto tile_row_ids = [&](int r, int& src, int& dst) {
+    src = -1;
+    dst = -1;
+    if (p.moe) {
+      if (r < p.moe_bs) {
+        const int id = p.sorted_ids[mt * p.moe_bs + r];
+        if (id < p.c_rows) {
+          src = id / p.top_k;
+          dst = id;
+        }
+      }
+    } else {
+      const int gr = mt * 16 + r;
+      if (gr < p.M) src = dst = gr;
+    }
+  };
+  // activation loads: lane -> row (lane >> 3) [+ 8 for the second load], 16-byte piece (lane & 7) of the
+  // stage's 128 bytes.  Rows past the end of the problem read the tile's first row; never stored.
+  const int ar = lane >> 3, ap = lane & 7;
+  const uint16_t* arow[2];
+  {
+    int src0, dst0;
+    tile_row_ids(0, src0, dst0);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      int src, dst;
+      tile_row_ids(ar + 8 * i, src, dst);
+      arow[i] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + ap * 8;
+    }
+  }
+  if (threadIdx.x < 16) {
+    int src, dst;
+    tile_row_ids(threadIdx.x, src, dst);
+    s_crow[threadIdx.x] = dst;
+  }
+
+  // ---- this wavefront's stages (pairs of k-steps)
+  const int st_b = split * p.ksteps_per_split / 2;
+  const int st_e = min(st_b + p.ksteps_per_split / 2, p.total_ksteps / 2);
+  const int per = (st_e - st_b + DNW - 1) / DNW;
+  const int w_b = min(st_b + wv * per, st_e), w_e = min(w_b + per, st_e);
+  const int nst = w_e - w_b;
+
+  // n-tile this lane reads (TN=128: 2ct+h, TN=64: ct); a missing second n-tile (N/64 odd) aliases n-tile 0
+  int nt;
+  if (TN == 128)
+    nt = (2 * ct + h) * 64 < p.N ? 2 * ct + h : 0;
+  else
+    nt = ct;
+  const int64_t b_row = (int64_t)p.N * 2;  // words per k-tile row
+  // TN=128: words th*4 .. +4 of the n-tile, th = 4c+g.  TN=64: words th*4 + 2h .. +2.
+  const uint32_t* bp = Bq + (int64_t)nt * 128 + (4 * c + g) * 4 + (TN == 64 ? 2 * h : 0) + (int64_t)(4 * w_b) * b_row;
+  // scales of the lane's columns: permuted position 8c + j, j = 2w + half; TN=64 covers w = 2h, 2h+1 only
+  const uint16_t* sp = Sc + (int64_t)nt * 64 + 8 * c + (TN == 64 ? 4 * h : 0);
+  const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
+
+  // wavefront-private LDS slab for the A bounce: [row 16][36 dwords]: 32 dwords = 8 pieces x 4, +4 pad
+  // (bank = 36*row + 4*piece + dword is conflict-free for the reads below).
+  constexpr int A_ROW = 36;
+  uint32_t* slab = (uint32_t*)smem + wv * (16 * A_ROW);
+  uint32_t* slab_wr = slab + ar * A_ROW + ap * 4;
+  const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
+
+  struct Stage {
+    bvec b[4];   // k-tiles 4s .. 4s+3
+    u32x4 a[2];  // rows ar, ar+8
+    bvec sc;     // scales (pairs half0|half1 per word)
+    uint32_t zq;
+    int gi;
+  };
+  Stage st[DD];
+
+  auto issue = [&](Stage& s, int sidx) {  // sidx: absolute stage index (2 k-steps = 4 k-tiles = 64 K rows)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if constexpr (PERM) {
+        uint16_t e[8];
+        const uint16_t* row = arow[i] - ap * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = row[perm[sidx * 64 + ap * 8 + j]];
+        s.a[i] = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                       (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+      } else {
+        s.a[i] = *(const u32x4*)(arow[i] + sidx * 64);
+      }
+    }
+    const int gi = CHANNEL ? 0 : (2 * sidx) / p.group_ksteps;
+    s.gi = gi;
+    if (!CHANNEL)
+      s.sc = *(const bvec*)(sp + (int64_t)gi * p.N);
+    else
+      s.sc = bvec(0);
+    if (ZP) s.zq = zp[(int64_t)gi * (p.N >> 3)];
+    const uint32_t* q = bp + (int64_t)(4 * (sidx - w_b)) * b_row;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s.b[t] = __builtin_nontemporal_load((const bvec*)(q + t * b_row));
+  };
+
+  f32x4 acc[W][2], tmp[W][2];
+  f32x4 rs = {0, 0, 0, 0};
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    acc[w][0] = f32x4{0, 0, 0, 0};
+    acc[w][1] = f32x4{0, 0, 0, 0};
+    tmp[w][0] = f32x4{0, 0, 0, 0};
+    tmp[w][1] = f32x4{0, 0, 0, 0};
+  }
+  int cur_gi = -1;
+  bool fresh = true;
+  bvec cur_sc;
+  uint32_t cur_zq = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) cur_sc[w] = 0;
+
+  // acc += s * (tmp - e * rs),  e = E + z  (HI_TRICK: the bias operand already carries E + 8, e = 1)
+  auto fold = [&]() {
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      float s0 = 1.0f, s1 = 1.0f;
+      if (!CHANNEL) {
+        const uint32_t sw = cur_sc[w];
+        s0 = (DT == DT_F16) ? f16_lo_f32(sw) : bf16_lo_f32(sw);
+        s1 = (DT == DT_F16) ? f16_hi_f32(sw) : bf16_hi_f32(sw);
+      }
+      float e0 = 1.0f, e1 = 1.0f;
+      if constexpr (!HI_TRICK) {
+        const float E = (DT == DT_F16) ? 1024.0f : 128.0f;
+        const int wa = (TN == 64) ? 2 * h + w : w;  // absolute word index of the n-tile
+        e0 = E + (ZP ? (float)((cur_zq >> (4 * wa)) & 0xf) : 8.0f);
+        e1 = E + (ZP ? (float)((cur_zq >> (4 * wa + 16)) & 0xf) : 8.0f);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float d0 = __builtin_fmaf(-e0, rs[r], tmp[w][0][r]);
+        const float d1 = __builtin_fmaf(-e1, rs[r], tmp[w][1][r]);
+        acc[w][0][r] = __builtin_fmaf(s0, d0, acc[w][0][r]);
+        acc[w][1][r] = __builtin_fmaf(s1, d1, acc[w][1][r]);
+      }
+    }
+  };
+
+  auto consume = [&](const Stage& s) {
+    if (s.gi != cur_gi) {
+      if (cur_gi >= 0) fold();
+      cur_gi = s.gi;
+      cur_sc = s.sc;
+      cur_zq = s.zq;
+      fresh = true;
+    }
+    // A bounce: natural [row][128 B] layout in, MFMA operand (row m, K pairs 8s+2g) out
+    *(u32x4*)slab_wr = s.a[0];
+    *(u32x4*)(slab_wr + 8 * A_ROW) = s.a[1];
+    u32x4 af[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const uint32_t* q = slab_rd + kk * 16;
+      af[kk] = u32x4{q[0], q[4], q[8], q[12]};
+    }
+    u32x4 vb;  // B operand of the bias-term MFMA
+    if constexpr (HI_TRICK) {
+      const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        af[kk][1] = as_u32(as_h2(af[kk][1]) * sixteenth);
+        af[kk][3] = as_u32(as_h2(af[kk][3]) * sixteenth);
+      }
+      vb = u32x4{0x64086408u, 0x64806480u, 0x64086408u, 0x64806480u};  // 1032 | 1152 = 16 * 72
+    } else {
+      const uint32_t one = (DT == DT_F16) ? 0x3c003c00u : 0x3f803f80u;
+      vb = u32x4{one, one, one, one};
+    }
+    const f32x4 zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      u32x4 o[W][2];
+#pragma unroll
+      for (int w = 0; w < W; ++w) raw_pair<DT, HI_TRICK>(s.b[2 * kk][w], s.b[2 * kk + 1][w], o[w][0], o[w][1]);
+      if (kk == 0 && fresh) {
+        rs = mfma16x16x32<DT>(af[kk], vb, zero);
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          tmp[w][0] = mfma16x16x32<DT>(af[kk], o[w][0], zero);
+          tmp[w][1] = mfma16x16x32<DT>(af[kk], o[w][1], zero);
+        }
+      } else {
+        rs = mfma16x16x32<DT>(af[kk], vb, rs);
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          tmp[w][0] = mfma16x16x32<DT>(af[kk], o[w][0], tmp[w][0]);
+          tmp[w][1] = mfma16x16x32<DT>(af[kk], o[w][1], tmp[w][1]);
+        }
+      }
+    }
+    fresh = false;
+  };
+
+  // ---- software pipeline over stages (see the skinny kernel for why the scheduling barriers are there)
+  int done = 0;
+  if (nst >= DD) {
+#pragma unroll
+    for (int j = 0; j < DD; ++j) issue(st[j], w_b + j);
+    for (; done + 2 * DD <= nst; done += DD) {
+#pragma unroll
+      for (int j = 0; j < DD; ++j) {
+        consume(st[j]);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(st[j], w_b + done + j + DD);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < DD; ++j)
+      if (j < nst) issue(st[j], w_b + j);
+  }
+#pragma unroll 1
+  for (; done < nst; done += DD) {
+#pragma unroll
+    for (int j = 0; j < DD; ++j) {
+      const int i = done + j;
+      if (i < nst) {
+        consume(st[j]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + DD < nst) issue(st[j], w_b + i + DD);
+      }
+    }
+  }
+  if (cur_gi >= 0) fold();
+
+  // ------------------------------------------------------------------------------ epilogue
+  // red[wave][row 16][RS floats]; column position inside the tile: TN=128: 72h + 16w + 8half + c
+  // (real column 64h + 16w + 8half + c), TN=64: 40h + 16w + 8half + c (real column 32h + 16w + 8half + c).
+  float* red = (float*)smem;
+  const int t = threadIdx.x;
+  constexpr int CPT = TN / 32;          // consecutive columns per thread in the final phase (4 or 2)
+  const int fr = t >> 5;                // tile row
+  const int fc = (t & 31) * CPT;        // first column inside the tile
+  const int fpos = (TN == 128) ? fc + (fc >= 64 ? 8 : 0) : fc + (fc >= 32 ? 8 : 0);
+  const int ncol = ct * TN + fc;
+  const bool fcol_ok = ncol < p.N;
+  const bool single = p.splits == 1;
+  float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (16 * TN);
+
+  auto finalize = [&](float* v) {
+    const int crow = s_crow[fr];
+    if (crow < 0 || !fcol_ok) return;
+    const int base = ncol & ~31, cl = ncol & 31;
+    if (CHANNEL) {
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        v[j] *= (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+    }
+    if (bias) {
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        v[j] += (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+    if (p.mul_topk) {
+      const float tw = p.topk_w[crow];
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) v[j] *= tw;
+    }
+    uint16_t* dst = (uint16_t*)p.C + (int64_t)crow * p.N + ncol;
+#pragma unroll
+    for (int j = 0; j < CPT; j += 2)
+      *(uint32_t*)(dst + j) = (DT == DT_F16) ? pack_f16(v[j], v[j + 1]) : pack_bf16(v[j], v[j + 1]);
+  };
+
+  __syncthreads();  // A bounce slabs no longer read
+  {
+    float* mine = red + wv * (16 * RS);
+    constexpr int HS = (TN == 128) ? 72 : 40;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mine[(4 * g + r) * RS + HS * h + 16 * w + 8 * hf + c] = acc[w][hf][r];
+  }
+  __syncthreads();
+  float v[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) v[j] = 0.0f;
+#pragma unroll
+  for (int ww = 0; ww < DNW; ++ww) {
+    const float* src = red + ww * (16 * RS) + fr * RS + fpos;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) v[j] += src[j];
+  }
+  if (single) {
+    finalize(v);
+    return;
+  }
+  if (s_crow[fr] >= 0) {
+#pragma unroll
+    for (int j = 0; j < CPT; j += 2) store_coherent2(my_part + fr * TN + fc + j, v[j], v[j + 1]);
+  }
+  // ---- cross-workgroup reduction: the last split to arrive sums all partials in split order
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (t == 0) {
+    const int old = __hip_atomic_fetch_add(&p.locks[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == p.splits - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  if (s_crow[fr] >= 0) {
+    const float* parts = p.ctmp + (int64_t)tile * p.splits * (16 * TN) + fr * TN + fc;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) v[j] = 0.0f;
+    for (int s = 0; s < p.splits; ++s) {
+#pragma unroll
+      for (int j = 0; j < CPT; j += 2) {
+        float a0, a1;
+        load_coherent2(parts + (int64_t)s * (16 * TN) + j, a0, a1);
+        v[j] += a0;
+        v[j + 1] += a1;
+      }
+    }
+    finalize(v);
+  }
+  if (t == 0) __hip_atomic_store(&p.locks[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------------------------------------------ host side
+typedef void (*decode_fn)(const KParams);
+
+template <int DT, bool PERM, int TN>
+static decode_fn pick3(bool zp, bool channel) {
+  if (zp) return channel ? decode_kernel<DT, true, true, PERM, TN> : decode_kernel<DT, true, false, PERM, TN>;
+  return channel ? decode_kernel<DT, false, true, PERM, TN> : decode_kernel<DT, false, false, PERM, TN>;
+}
+template <int DT, bool PERM>
+static decode_fn pick2(int tn, bool zp, bool channel) {
+  return tn == 64 ? pick3<DT, PERM, 64>(zp, channel) : pick3<DT, PERM, 128>(zp, channel);
+}
+
+static decode_fn pick_decode(int dt, bool perm, int tn, bool zp, bool channel) {
+  if (dt == DT_F16) return perm ? pick2<DT_F16, true>(tn, zp, channel) : pick2<DT_F16, false>(tn, zp, channel);
+  return perm ? pick2<DT_BF16, true>(tn, zp, channel) : pick2<DT_BF16, false>(tn, zp, channel);
+}
+
+int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
+  const bool zp = a->b_zeros != nullptr;
+  decode_fn fn = pick_decode(a->dtype, pl.use_perm, pl.tn, zp, pl.gm == GM_CHANNEL);
+  KParams p = make_kparams(a, pl);
+  const int smem = pl.tn == 64 ? DecodeCfg<64>::SMEM : DecodeCfg<128>::SMEM;
+  if (smem > 64 * 1024) {
+    static const void* allowed[32];
+    static int n_allowed = 0;
+    bool seen = false;
+    for (int i = 0; i < n_allowed; ++i) seen |= allowed[i] == (const void*)fn;
+    if (!seen) {
+      W4A16_HIP(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+      if (n_allowed < 32) allowed[n_allowed++] = (const void*)fn;
+    }
+  }
+  const int64_t grid = (int64_t)pl.tiles * pl.splits;
+  if (grid <= 0) return 0;
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(DNW * 64), smem, stream, p);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace w4a16

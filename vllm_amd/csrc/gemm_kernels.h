@@ -1,0 +1,112 @@
+// Kernel parameter block and cross-workgroup helpers shared by the W4A16 GEMM kernels.
+#pragma once
+#include "gemm_plan.h"
+
+namespace w4a16 {
+
+struct KParams {
+  const void* A;
+  int64_t lda;
+  void* C;
+  const uint32_t* B;
+  const void* S;
+  const uint32_t* Z;
+  const int32_t* gidx;
+  const int32_t* perm;
+  const void* bias;
+  float* ctmp;
+  int32_t* locks;
+  int M;       // rows of A
+  int c_rows;  // rows of C (M, or M*top_k for MoE)
+  int N, K;
+  int group_ksteps;  // GM_GROUPED: group_size / 32
+  int ncp;           // column pairs = ceil(N / 128)
+  int splits, ksteps_per_split, total_ksteps;
+  int xcd_map;
+  int fix_mode;  // debugging switches (0 in production)
+  int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
+  // MoE
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* ntpp;
+  const float* topk_w;
+  int moe, moe_bs, top_k, mul_topk;
+  int64_t b_estride, s_estride, z_estride, k_estride, n_estride;  // per-expert strides (elements)
+};
+
+// Split-K partials cross XCDs (each XCD has its own L2).  A plain store stays dirty in the writer's L2,
+// and an agent-scope release fence (an L2 write-back) costs ~0.5 us per workgroup, serialised per L2.
+// Instead every partial is written with relaxed agent-scope atomic stores (global_store ... sc1: written
+// through to the device-coherent level) and read back with agent-scope loads (sc1: never served from a
+// non-coherent line), 8 bytes at a time.  The writer waits for its stores (s_waitcnt) before it counts
+// itself as arrived; the reader is whoever sees the last arrival.
+__device__ __forceinline__ void store_coherent2(float* ptr, float f0, float f1) {
+  using u64 = unsigned long long;
+  const u64 a = (u64)__builtin_bit_cast(uint32_t, f0) | ((u64)__builtin_bit_cast(uint32_t, f1) << 32);
+  __hip_atomic_store((u64*)ptr, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_coherent(float* ptr, f32x4 v, int /*mode*/ = 0) {
+  // (elements are copied to scalars first: bit-casting a vector element directly reads element 0)
+  const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
+  store_coherent2(ptr, f0, f1);
+  store_coherent2(ptr + 2, f2, f3);
+}
+__device__ __forceinline__ void load_coherent2(const float* ptr, float& f0, float& f1) {
+  using u64 = unsigned long long;
+  const u64 a = __hip_atomic_load((const u64*)ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  f0 = __builtin_bit_cast(float, (uint32_t)a);
+  f1 = __builtin_bit_cast(float, (uint32_t)(a >> 32));
+}
+__device__ __forceinline__ f32x4 load_coherent(const float* ptr, int /*mode*/ = 0) {
+  float f0, f1, f2, f3;
+  load_coherent2(ptr, f0, f1);
+  load_coherent2(ptr + 2, f2, f3);
+  return f32x4{f0, f1, f2, f3};
+}
+
+// Host: translate the C-ABI arguments and the launch plan into the kernel parameter block.
+inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
+  const bool moe = (a->flags & W4A16_F_MOE) != 0;
+  KParams p{};
+  p.A = a->a;
+  p.lda = a->lda;
+  p.C = a->c;
+  p.B = a->b_q_weight;
+  p.S = a->b_scales;
+  p.Z = a->b_zeros;
+  p.gidx = pl.gm == GM_GIDX ? a->g_idx : nullptr;
+  p.perm = pl.use_perm ? a->perm : nullptr;
+  p.bias = a->b_bias;
+  p.ctmp = a->c_tmp;
+  p.locks = a->workspace;
+  p.M = (int)a->size_m;
+  p.c_rows = (int)(moe ? a->size_m * a->top_k : a->size_m);
+  p.N = (int)a->size_n;
+  p.K = (int)a->size_k;
+  p.group_ksteps = pl.group_ksteps;
+  p.ncp = pl.ncp;
+  p.splits = pl.splits;
+  p.ksteps_per_split = pl.kps;
+  p.total_ksteps = pl.total_ksteps;
+  p.xcd_map = pl.xcd_map;
+  p.fix_mode = 0;
+  p.tn = pl.tn;
+  p.sorted_ids = a->sorted_token_ids;
+  p.expert_ids = a->expert_ids;
+  p.ntpp = a->num_tokens_past_padded;
+  p.topk_w = a->topk_weights;
+  p.moe = moe;
+  p.moe_bs = a->moe_block_size;
+  p.top_k = moe ? a->top_k : 1;
+  p.mul_topk = moe && (a->flags & W4A16_F_MUL_TOPK_WEIGHTS);
+  p.b_estride = (a->size_k / 16) * (2 * a->size_n);
+  p.s_estride = a->num_groups * a->size_n;
+  p.z_estride = a->num_groups * (a->size_n / 8);
+  p.k_estride = a->size_k;
+  p.n_estride = a->size_n;
+  return p;
+}
+
+constexpr int RED_RS = 148;  // row stride (floats) of the 128-column reduction slab (4 mod 16: conflict-free)
+
+}  // namespace w4a16

@@ -22,81 +22,16 @@
 // once per column pair (from L2), split partials move 2 * splits * M * N * 4 bytes.
 #include <stdlib.h>
 
-#include "gemm_plan.h"
+#include "gemm_kernels.h"
 
 namespace w4a16 {
 
-struct KParams {
-  const void* A;
-  int64_t lda;
-  void* C;
-  const uint32_t* B;
-  const void* S;
-  const uint32_t* Z;
-  const int32_t* gidx;
-  const int32_t* perm;
-  const void* bias;
-  float* ctmp;
-  int32_t* locks;
-  int M;       // rows of A
-  int c_rows;  // rows of C (M, or M*top_k for MoE)
-  int N, K;
-  int group_ksteps;  // GM_GROUPED: group_size / 32
-  int ncp;           // column pairs = ceil(N / 128)
-  int splits, ksteps_per_split, total_ksteps;
-  int xcd_map;
-  int fix_mode;
-  // MoE
-  const int32_t* sorted_ids;
-  const int32_t* expert_ids;
-  const int32_t* ntpp;
-  const float* topk_w;
-  int moe, moe_bs, top_k, mul_topk;
-  int64_t b_estride, s_estride, z_estride, k_estride, n_estride;  // per-expert strides (elements)
-};
-
-// Split partials cross XCDs (each XCD has its own L2).  A plain store stays dirty in the writer's L2
-// and an agent-scope release fence (L2 write-back) costs ~0.5 us per workgroup, serialised per L2.
-// Instead every partial word is written with an agent-scope atomic exchange, which is performed at
-// the device-coherent level, and read back with agent-scope loads (sc1: bypass non-coherent lines).
-__device__ __forceinline__ void store_coherent(float* ptr, f32x4 v, int mode) {
-  using u64 = unsigned long long;
-  // (elements are copied to scalars first: bit-casting a vector element directly reads element 0)
-  const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
-  const u64 a = (u64)__builtin_bit_cast(uint32_t, f0) | ((u64)__builtin_bit_cast(uint32_t, f1) << 32);
-  const u64 b = (u64)__builtin_bit_cast(uint32_t, f2) | ((u64)__builtin_bit_cast(uint32_t, f3) << 32);
-  if (mode == 3) {
-    __hip_atomic_store((u64*)ptr, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store((u64*)ptr + 1, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  } else if (mode == 0) {
-    __hip_atomic_store((u64*)ptr, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store((u64*)ptr + 1, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  } else {
-    __hip_atomic_exchange((u64*)ptr, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_exchange((u64*)ptr + 1, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-__device__ __forceinline__ f32x4 load_coherent(const float* ptr, int mode) {
-  using u64 = unsigned long long;
-  u64 a, b;
-  if (mode == 3) {
-    a = __hip_atomic_load((const u64*)ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    b = __hip_atomic_load((const u64*)ptr + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  } else {
-    a = __hip_atomic_load((const u64*)ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    b = __hip_atomic_load((const u64*)ptr + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  return f32x4{__builtin_bit_cast(float, (uint32_t)a), __builtin_bit_cast(float, (uint32_t)(a >> 32)),
-               __builtin_bit_cast(float, (uint32_t)b), __builtin_bit_cast(float, (uint32_t)(b >> 32))};
-}
-
 constexpr int NW = 8;        // wavefronts per workgroup
-constexpr int RED_RS = 148;  // row stride (floats) of the reduction slab; see epilogue
 
 template <int MB>
 struct SkinnyCfg {
-  static constexpr int D = (MB >= 4) ? 3 : (MB == 2 ? 6 : 8);  // k-steps in flight per wavefront
-  static constexpr int SMEM = NW * 16 * RED_RS * 4;             // reduction slab only
+  static constexpr int D = (MB >= 4) ? 3 : 6;  // k-steps in flight per wavefront
+  static constexpr int SMEM = NW * 16 * RED_RS * 4;  // reduction slab; its head doubles as the A bounce slabs
 };
 
 
@@ -105,6 +40,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   constexpr int BM = 16 * MB;
   constexpr int D = SkinnyCfg<MB>::D;
   constexpr bool UNIT = (GM == GM_CHANNEL);
+  // Decode tiles (one m-block) keep the weights as raw magic numbers E+q in the MFMA and apply
+  // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
+  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX);
+  constexpr bool HI_TRICK = FOLD && (DT == DT_F16) && !ZP;
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
   __shared__ int s_last;
@@ -112,7 +51,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const int lane = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
-  const int am = lane & 15;  // activation row inside an m-block (MFMA A operand row)
+  const int am = lane >> 2;  // activation row (inside an m-block) this lane loads
+  const int ap = lane & 3;   // ... and which 16-byte piece of the k-step's 64 bytes
 
   int tile, split;
   {
@@ -173,7 +113,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     for (int mb = 0; mb < MB; ++mb) {
       int src, dst;
       tile_row_ids(mb * 16 + am, src, dst);
-      arow[mb] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + g * 8;
+      arow[mb] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + ap * 8;
     }
   }
   if (threadIdx.x < BM) {
@@ -187,7 +127,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const int ks_e = min(ks_b + p.ksteps_per_split, p.total_ksteps);
   const int per = (ks_e - ks_b + NW - 1) / NW;
   const int w_b = min(ks_b + wv * per, ks_e), w_e = min(w_b + per, ks_e);
-  const int nks = (p.fix_mode == 12 || p.fix_mode == 13) ? 0 : w_e - w_b;
+  const int nks = w_e - w_b;
 
   // lanes of an n-tile past the end of N (odd number of n-tiles) read n-tile 0; their columns are never stored
   const int nt = (2 * cp + h) * 64 < p.N ? 2 * cp + h : 0;
@@ -197,9 +137,15 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
 
-  // Activations: lane (row am, piece g) loads the 16 bytes A[row][32ks + 8g .. +8) = K pairs 8g+2q, q=0..3.
-  // The MFMA lane (row, g) needs pair 8s+2g for s=0..3, i.e. register g of the lane 16s+row: a 4x4
-  // transpose between the four 16-lane groups and the four registers, done with permlane swaps.
+  // Activations: lane (row am = l>>2, piece ap = l&3) loads the 16 bytes A[row][32ks + 8ap .. +8), so one
+  // 16-lane pass of the load covers 4 rows x 64 contiguous bytes.  The MFMA lane (row m = l&15, g = l>>4)
+  // needs K pairs 8s+2g, s = 0..3, i.e. dword g of pieces 0..3 of row m: the 1 KiB is bounced through a
+  // wavefront-private LDS slab laid out [row][piece][dword] with an 80-byte row stride (conflict-free:
+  // bank = 20*row + 4*piece + dword).  LDS ops of one wavefront execute in order, so no barrier is needed.
+  constexpr int A_ROW = 20;  // dwords per row (16 + 4 pad)
+  uint32_t* slab = (uint32_t*)smem + wv * (MB * 16 * A_ROW);
+  uint32_t* slab_wr = slab + am * A_ROW + ap * 4;
+  const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
   struct Stage {
     u32x4 b0, b1, sc;
     u32x4 a[MB];
@@ -214,9 +160,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     for (int mb = 0; mb < MB; ++mb) {
       if constexpr (PERM) {
         uint16_t e[8];
-        const uint16_t* row = arow[mb] - g * 8;
+        const uint16_t* row = arow[mb] - ap * 8;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = row[perm[ks * 32 + g * 8 + j]];
+        for (int j = 0; j < 8; ++j) e[j] = row[perm[ks * 32 + ap * 8 + j]];
         s.a[mb] = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
                         (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
       } else {
@@ -246,18 +192,90 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       acc[mb][w][1] = f32x4{0, 0, 0, 0};
     }
 
+  // ---- fold scheme state (FOLD only): tmp = sum_k a_k (E + q_k) over the k-steps of the current group,
+  // rs = sum_k a_k * v_k, the matching bias term (v = E + 8 for uint4b8 in the HI_TRICK form, else 1).
+  f32x4 tmp[4][2];
+  f32x4 rs = {0, 0, 0, 0};
+  int cur_gi = -1;
+  bool fresh = true;
+  u32x4 cur_sc = {0, 0, 0, 0};
+  uint32_t cur_zq = 0;
+  // acc += s * (tmp - (E + z) * rs)   [HI_TRICK: acc += s * (tmp - rs)]
+  auto fold = [&]() {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float s0 = 1.0f, s1 = 1.0f;
+      if (GM != GM_CHANNEL) {
+        s0 = (DT == DT_F16) ? f16_lo_f32(cur_sc[w]) : bf16_lo_f32(cur_sc[w]);
+        s1 = (DT == DT_F16) ? f16_hi_f32(cur_sc[w]) : bf16_hi_f32(cur_sc[w]);
+      }
+      float e0 = 1.0f, e1 = 1.0f;
+      if constexpr (!HI_TRICK) {
+        const float E = (DT == DT_F16) ? 1024.0f : 128.0f;
+        e0 = E + (ZP ? (float)((cur_zq >> (4 * w)) & 0xf) : 8.0f);
+        e1 = E + (ZP ? (float)((cur_zq >> (4 * w + 16)) & 0xf) : 8.0f);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float d0 = __builtin_fmaf(-e0, rs[r], tmp[w][0][r]);
+        const float d1 = __builtin_fmaf(-e1, rs[r], tmp[w][1][r]);
+        acc[0][w][0][r] = __builtin_fmaf(s0, d0, acc[0][w][0][r]);
+        acc[0][w][1][r] = __builtin_fmaf(s1, d1, acc[0][w][1][r]);
+      }
+    }
+  };
+
   auto consume = [&](const Stage& s, int ks) {
     u32x4 af[MB];
+    {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) *(u32x4*)(slab_wr + mb * 16 * A_ROW) = s.a[mb];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      uint32_t r0 = s.a[mb][0], r1 = s.a[mb][1], r2 = s.a[mb][2], r3 = s.a[mb][3];
-      typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-      u2 t;
-      t = __builtin_amdgcn_permlane32_swap(r0, r2, false, false); r0 = t[0]; r2 = t[1];
-      t = __builtin_amdgcn_permlane32_swap(r1, r3, false, false); r1 = t[0]; r3 = t[1];
-      t = __builtin_amdgcn_permlane16_swap(r0, r1, false, false); r0 = t[0]; r1 = t[1];
-      t = __builtin_amdgcn_permlane16_swap(r2, r3, false, false); r2 = t[0]; r3 = t[1];
-      af[mb] = u32x4{r0, r1, r2, r3};
+      const uint32_t* q = slab_rd + mb * 16 * A_ROW;
+      af[mb] = u32x4{q[0], q[4], q[8], q[12]};
+    }
+    }
+    if constexpr (FOLD) {
+      if (s.gi != cur_gi) {
+        if (cur_gi >= 0) fold();
+        cur_gi = s.gi;
+        cur_sc = s.sc;
+        cur_zq = s.zq;
+        fresh = true;
+      }
+      u32x4 vb;  // B operand of the bias-term MFMA
+      if constexpr (HI_TRICK) {
+        // activations of the high-nibble K rows (slots 1, 3) are scaled by 1/16 (exact)
+        const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+        af[0][1] = as_u32(as_h2(af[0][1]) * sixteenth);
+        af[0][3] = as_u32(as_h2(af[0][3]) * sixteenth);
+        vb = u32x4{0x64086408u, 0x64806480u, 0x64086408u, 0x64806480u};  // 1032, 1152 = 16 * 72
+      } else {
+        const uint32_t one = (DT == DT_F16) ? 0x3c003c00u : 0x3f803f80u;
+        vb = u32x4{one, one, one, one};
+      }
+      u32x4 o[4][2];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) raw_pair<DT, HI_TRICK>(s.b0[w], s.b1[w], o[w][0], o[w][1]);
+      const f32x4 zero = {0, 0, 0, 0};
+      if (fresh) {
+        fresh = false;
+        rs = mfma16x16x32<DT>(af[0], vb, zero);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          tmp[w][0] = mfma16x16x32<DT>(af[0], o[w][0], zero);
+          tmp[w][1] = mfma16x16x32<DT>(af[0], o[w][1], zero);
+        }
+      } else {
+        rs = mfma16x16x32<DT>(af[0], vb, rs);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          tmp[w][0] = mfma16x16x32<DT>(af[0], o[w][0], tmp[w][0]);
+          tmp[w][1] = mfma16x16x32<DT>(af[0], o[w][1], tmp[w][1]);
+        }
+      }
+      return;
     }
     if (GM == GM_GIDX && !s.uni) {
       // group boundary inside the k-step: fetch the scale row of every K-row separately
@@ -345,6 +363,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     }
   }
 
+  if constexpr (FOLD) {
+    if (cur_gi >= 0) fold();
+  }
+
   // ------------------------------------------------------------------------------ epilogue
   // Reduction slab: red[wave][row 0..15][RED_RS floats]; column position of real column
   // (h, w, half, c) is 72h + 16w + 8half + c.  With RED_RS = 148 (= 4 mod 16) the 64 lanes of one
@@ -393,7 +415,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    if (mb) __syncthreads();  // previous m-block's slab no longer read
+    __syncthreads();  // A bounce slabs / previous m-block's slab no longer read
     {
       float* mine = red + wv * (16 * RED_RS);
 #pragma unroll
@@ -412,10 +434,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     if (single)
       finalize(r, v);
     else if (s_crow[r] >= 0)
-      store_coherent(my_part + r * 128 + fc4, v, p.fix_mode);
+      store_coherent(my_part + r * 128 + fc4, v);
   }
   if (single) return;
-  if (p.fix_mode == 10 || p.fix_mode == 13) return;
 
   // ---- cross-workgroup reduction: the last split to arrive sums all partials in split order.
   // The wait makes every partial of this workgroup complete before its arrival is counted.
@@ -434,7 +455,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     if (s_crow[r] < 0) continue;
     f32x4 v = {0, 0, 0, 0};
     for (int s = 0; s < p.splits; ++s)
-      v += load_coherent(parts + (int64_t)s * (BM * 128) + r * 128 + fc4, p.fix_mode);
+      v += load_coherent(parts + (int64_t)s * (BM * 128) + r * 128 + fc4);
     finalize(r, v);
   }
   if (t == 0) __hip_atomic_store(&p.locks[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -479,46 +500,7 @@ int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
   const bool zp = a->b_zeros != nullptr;
   skinny_fn fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm);
   if (!fn) return fail(W4A16_EINVAL, "unsupported kernel variant");
-  const bool moe = (a->flags & W4A16_F_MOE) != 0;
-  KParams p{};
-  p.A = a->a;
-  p.lda = a->lda;
-  p.C = a->c;
-  p.B = a->b_q_weight;
-  p.S = a->b_scales;
-  p.Z = a->b_zeros;
-  p.gidx = pl.gm == GM_GIDX ? a->g_idx : nullptr;
-  p.perm = pl.use_perm ? a->perm : nullptr;
-  p.bias = a->b_bias;
-  p.ctmp = a->c_tmp;
-  p.locks = a->workspace;
-  p.M = (int)a->size_m;
-  p.c_rows = (int)(moe ? a->size_m * a->top_k : a->size_m);
-  p.N = (int)a->size_n;
-  p.K = (int)a->size_k;
-  p.group_ksteps = pl.group_ksteps;
-  p.ncp = pl.ncp;
-  p.splits = pl.splits;
-  p.ksteps_per_split = pl.kps;
-  p.total_ksteps = pl.total_ksteps;
-  p.xcd_map = pl.xcd_map;
-  {
-    static const char* fm = getenv("W4A16_FIXMODE");
-    p.fix_mode = fm ? atoi(fm) : 2;
-  }
-  p.sorted_ids = a->sorted_token_ids;
-  p.expert_ids = a->expert_ids;
-  p.ntpp = a->num_tokens_past_padded;
-  p.topk_w = a->topk_weights;
-  p.moe = moe;
-  p.moe_bs = a->moe_block_size;
-  p.top_k = moe ? a->top_k : 1;
-  p.mul_topk = moe && (a->flags & W4A16_F_MUL_TOPK_WEIGHTS);
-  p.b_estride = (a->size_k / 16) * (2 * a->size_n);
-  p.s_estride = a->num_groups * a->size_n;
-  p.z_estride = a->num_groups * (a->size_n / 8);
-  p.k_estride = a->size_k;
-  p.n_estride = a->size_n;
+  KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);
   if (smem > 64 * 1024) {
     // more than 64 KiB of dynamic LDS has to be allowed per kernel function; do it once per function
