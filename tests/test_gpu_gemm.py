@@ -172,3 +172,54 @@ def test_llama_shapes_fp16(ops, dev, workspace, shape, m):
     out = run_gemm(ops, layer, a, dev, workspace)
     check_close(out, a, layer)
     assert int(workspace.abs().sum()) == 0
+
+
+# ------------------------------------------------------------------------- prefill (128-row tile) kernel
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("has_zp", [False, True])
+@pytest.mark.parametrize("group_size", [-1, 32, 128])
+def test_prefill_one_hot(ops, dev, workspace, dtype, has_zp, group_size):
+    """Identity activations through the large-M path: every dequantised weight row comes back bit-exact."""
+    size_k, size_n = 256, 576   # N = 4.5 column pairs: a partly filled 512-column tile and an odd n-tile
+    print(f"prefill one_hot dtype={dtype} zp={has_zp} g={group_size}", flush=True)
+    layer = make_layer(size_k, size_n, group_size, dtype, has_zp=has_zp, seed=21)
+    a = torch.eye(size_k, dtype=dtype)
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["gptq", "awq", "gptq_act_order", "channel"])
+@pytest.mark.parametrize("mnk", [(128, 512, 128), (129, 1088, 384), (300, 64, 1024), (1000, 2048, 2048)])
+def test_prefill_shapes(ops, dev, workspace, dtype, mode, mnk):
+    size_m, size_n, size_k = mnk
+    group = -1 if mode == "channel" else 128
+    if mode == "gptq_act_order" and size_k == group:
+        pytest.skip("act-order needs more than one group")
+    print(f"prefill {mode} dtype={dtype} m={size_m} n={size_n} k={size_k}", flush=True)
+    layer = make_layer(size_k, size_n, group, dtype, has_zp=(mode == "awq"), act_order=(mode == "gptq_act_order"),
+                       seed=size_m)
+    a = _a(size_m, size_k, dtype, dev, seed=3)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+
+
+def test_prefill_bias_and_strided_a(ops, dev, workspace):
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    size_m, size_k, size_n = 200, 512, 640
+    layer = make_layer(size_k, size_n, 128, torch.float16, seed=31)
+    g = torch.Generator().manual_seed(32)
+    a = torch.randn(size_m, size_k + 128, generator=g).half().to(dev)[:, 64:64 + size_k]
+    bias = torch.randn(size_n, generator=g).half().to(dev)
+    out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias))
+    check_close(out, a, layer, bias=bias)
+
+
+def test_prefill_llama_o_proj_bf16_awq(ops, dev, workspace):
+    """Configuration 3, o_proj: M = 4096, bf16, uint4 + zero points, group 128."""
+    size_m, size_k, size_n = 4096, 4096, 4096
+    print("prefill llama o_proj M=4096 bf16 awq", flush=True)
+    layer = make_layer(size_k, size_n, 128, torch.bfloat16, has_zp=True, seed=41, w_std=0.02, rule="benchmark")
+    a = _a(size_m, size_k, torch.bfloat16, dev, seed=42)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)

@@ -86,6 +86,29 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
 
+  pl.atmp_bytes = 0;
+  // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
+  static const int fat_min_m = env_int("W4A16_FAT_MIN_M", 128);
+  const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
+  if (!moe && a->size_m >= fat_min_m && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+      pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1) {
+    pl.kind = 2;
+    pl.tn = 512;
+    pl.mb = 8;
+    pl.bm = 128;
+    pl.mtiles = (int)ceil_div(a->size_m, 128);
+    pl.ncp = (int)ceil_div(a->size_n, 512);
+    const int64_t tiles = (int64_t)pl.mtiles * pl.ncp;
+    W4A16_CHECK(tiles < (1LL << 31) / 64, "too many tiles");
+    pl.tiles = (int)tiles;
+    pl.splits = 1;
+    pl.kps = pl.total_ksteps;
+    pl.xcd_map = 0;
+    pl.ctmp_bytes = 0;
+    if (pl.use_perm) pl.atmp_bytes = a->size_m * a->size_k * 2;
+    return 0;
+  }
+
   // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
   const bool decode_ok = pl.mb == 1 && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
                          (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
@@ -119,7 +142,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       const int64_t rounds = ceil_div(wgs, cus);
       double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
       if (rate > chip_rate) rate = chip_rate;
-      const double t = bytes / rate + (sp > 1 ? 2.8 + 0.05 * sp : 0.0);
+      // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
+      const double t_fix = sp > 1 ? 2.8 + sp * (double)(pl.bm * tn * 4) / 20e3 : 0.0;
+      const double t = bytes / rate + t_fix;
       if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, t};
     }
   }
@@ -154,7 +179,7 @@ extern "C" int64_t w4a16_gemm_scratch_bytes(const w4a16_gemm_args* args) {
   if (args->size_m == 0) return 0;
   Plan pl;
   if (int rc = make_plan(args, pl)) return rc;
-  return pl.ctmp_bytes;
+  return ((pl.ctmp_bytes + 255) & ~255LL) + pl.atmp_bytes;
 }
 
 extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
@@ -163,6 +188,21 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
   Plan pl;
   if (int rc = make_plan(args, pl)) return rc;
   if (pl.mtiles == 0) return 0;
-  if (pl.ctmp_bytes > 0) W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed", (long long)pl.ctmp_bytes);
+  if (pl.ctmp_bytes + pl.atmp_bytes > 0)
+    W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed",
+                (long long)(pl.ctmp_bytes + pl.atmp_bytes));
+  if (pl.kind == 2) {
+    w4a16_gemm_args b = *args;
+    if (pl.use_perm) {
+      // act-order in front of the prefill kernel: gather A's columns once (as the reference's permute_cols_kernel,
+      // csrc/quantization/gptq_marlin/gptq_marlin.cu:549-564), then run the plain grouped path on the copy
+      void* a_tmp = (char*)args->c_tmp + ((pl.ctmp_bytes + 255) & ~255LL);
+      if (int rc = w4a16_permute_cols(args->a, args->perm, a_tmp, args->size_m, args->size_k, args->lda, stream)) return rc;
+      b.a = a_tmp;
+      b.lda = args->size_k;
+      pl.use_perm = false;
+    }
+    return launch_fat(&b, pl, (hipStream_t)stream);
+  }
   return pl.kind == 1 ? launch_decode(args, pl, (hipStream_t)stream) : launch_skinny(args, pl, (hipStream_t)stream);
 }

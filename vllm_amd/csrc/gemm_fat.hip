@@ -1,0 +1,260 @@
+// W4A16 prefill GEMM for gfx950 (large M): C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias).
+//
+// Same operand layouts as the skinny kernel (gemm_common.h), tiled for the matrix cores:
+//   workgroup tile 128 rows x 512 columns, 4 wavefronts, each owning 128 rows x 128 columns (one column
+//   pair): 8 m-blocks x 8 MFMA column groups = 64 v_mfma_f32_16x16x32 per k-step, 256 fp32 accumulators
+//   per lane (one wavefront per SIMD, 512 registers).
+//   weights      each wavefront streams its own column pair global -> registers (128-bit loads) and
+//                dequantises it once per k-step (scale applied per element, so the B operand equals the
+//                reference's half(q - z) * half(s)); every dequantised operand feeds 8 MFMAs.
+//   activations  the workgroup stages 128 rows x 64 K (two k-steps, 128 contiguous bytes per row) into LDS,
+//                double buffered, already in MFMA fragment order, so an A operand is one conflict-free
+//                ds_read_b128; one barrier per two k-steps (128 MFMAs per wavefront).
+// MFMA work per byte of weights is 64x the decode kernel's; the bound is the matrix pipe, and the VALU work
+// of dequantisation (about 105 instructions per 64 MFMAs for fp16) is interleaved with them: the MFMAs run
+// word-major (16 per Marlin word), and as soon as a word's operands are dead the next k-step's word is
+// dequantised into the same registers.
+// Requirements (host-checked; otherwise the skinny kernel runs): dense op, K % 128 == 0, no per-row g_idx.
+#include "gemm_kernels.h"
+
+namespace w4a16 {
+
+constexpr int FB_MB = 8;     // m-blocks per wavefront
+constexpr int FB_BM = 128;   // rows per workgroup tile
+constexpr int FB_D = 4;      // weight k-steps in flight per wavefront
+constexpr int FB_ABUF = 2 * FB_MB * 64 * 16;  // bytes of one A buffer: 2 k-steps x 8 m-blocks x 64 lanes x 16 B
+constexpr int FB_SMEM = (2 * FB_ABUF > 4 * 16 * RED_RS * 4) ? 2 * FB_ABUF : 4 * 16 * RED_RS * 4;
+
+// In-place MFMA on an accumulator pinned to AGPRs.  With 256 accumulators per lane the register allocator
+// otherwise assigns different registers to an MFMA's source and destination accumulator and fills the loop
+// with v_accvgpr moves (more of them than dequantisation instructions).  Source C == destination is the form
+// the matrix pipe forwards without extra wait states; results are only read again after the main loop.
+template <int DT>
+__device__ __forceinline__ void mfma_inplace(f32x4& acc, const u32x4& a, const u32x4& b) {
+  if constexpr (DT == DT_F16)
+    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  else
+    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+template <int DT, bool ZP, bool CHANNEL>
+__global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
+  constexpr bool UNIT = CHANNEL;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
+
+  // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
+  const int mtiles = (p.M + FB_BM - 1) / FB_BM;
+  const int mt = blockIdx.x % mtiles, nt4 = blockIdx.x / mtiles;
+  const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
+  const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
+  const int row0 = mt * FB_BM;
+
+  // ---- weights of this wavefront
+  const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
+  const int64_t b_row = p.N >> 1;
+  const u32x4* bp = (const u32x4*)p.B + nt * 32 + (4 * c + g);
+  const int64_t s_row = p.N >> 3;
+  const u32x4* sp = (const u32x4*)p.S + nt * 8 + c;
+  const uint32_t* zp = ZP ? p.Z + nt * 8 + c : nullptr;
+
+  // ---- activation staging: thread t loads piece (t & 7) of rows (t >> 3) + 32 i, i = 0..3
+  const int piece = t & 7;
+  const uint16_t* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int r = row0 + (t >> 3) + 32 * i;
+    if (r >= p.M) r = p.M - 1;  // rows past the end replicate the last row; never stored
+    arow[i] = (const uint16_t*)p.A + (int64_t)r * p.lda + piece * 8;
+  }
+  // LDS A layout: [buffer][k-step 2][m-block 8][lane 64][4 dwords]; the 16 bytes of (row, piece) are the K
+  // pairs 8*pp + 2q (pp = piece & 3), which belong to lane (q*16 + row%16), dword pp, of k-step piece >> 2.
+  uint32_t* lds = (uint32_t*)smem;
+  int a_wr[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (t >> 3) + 32 * i;
+    a_wr[i] = (((piece >> 2) * FB_MB + (r >> 4)) * 64 + (r & 15)) * 4 + (piece & 3);
+  }
+  u32x4 areg[4];
+  // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
+  //  keeps the main loop free of branches, so the compiler can overlap LDS reads and dequantisation with MFMAs)
+  auto load_a = [&](int chunk) {
+    chunk = min(chunk, p.total_ksteps / 2 - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
+  };
+  auto store_a = [&](int buf) {
+    uint32_t* dst = lds + buf * (FB_ABUF / 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dst[a_wr[i] + q * 64] = areg[i][q];
+    }
+  };
+
+  struct Stage {
+    u32x4 b0, b1, sc;
+    uint32_t zq;
+  };
+  Stage st[FB_D];
+  auto issue = [&](Stage& s, int ks) {
+    ks = min(ks, p.total_ksteps - 1);
+    int gi = 0;
+    if (!CHANNEL) gi = ks / p.group_ksteps;
+    if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
+    if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    s.b0 = bp[(int64_t)(2 * ks) * b_row];
+    s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+  };
+  auto dequant_word = [&](const Stage& s, int w, u32x4& o0, u32x4& o1) {
+    uint32_t z0 = 8, z1 = 8;
+    if (ZP) {
+      z0 = (s.zq >> (4 * w)) & 0xf;
+      z1 = (s.zq >> (4 * w + 16)) & 0xf;
+    }
+    const ColConst<DT> cc = make_col_const<DT, UNIT>(CHANNEL ? 0u : s.sc[w], z0, z1);
+    dequant_pair<DT, UNIT>(s.b0[w], s.b1[w], cc, o0, o1);
+  };
+
+  f32x4 acc[FB_MB][4][2];
+#pragma unroll
+  for (int mb = 0; mb < FB_MB; ++mb)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      acc[mb][w][0] = f32x4{0, 0, 0, 0};
+      acc[mb][w][1] = f32x4{0, 0, 0, 0};
+    }
+
+  const int total = p.total_ksteps;  // multiple of 4 (K % 128 == 0)
+  const int nchunks = total / 2;
+
+  // ---- prologue
+  load_a(0);
+#pragma unroll
+  for (int j = 0; j < FB_D; ++j) issue(st[j], j);
+  store_a(0);
+  u32x4 ocur[4][2];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) dequant_word(st[0], w, ocur[w][0], ocur[w][1]);
+  __syncthreads();
+
+  // One k-step: 64 MFMAs on `ocur`, interleaved with the dequantisation of the next k-step's words.
+  auto kstep = [&](int buf, int kk, const Stage& nxt) {
+    const u32x4* abase = (const u32x4*)(lds + buf * (FB_ABUF / 4)) + (kk * FB_MB) * 64 + lane;
+    u32x4 af[FB_MB];
+#pragma unroll
+    for (int mb = 0; mb < FB_MB; ++mb) af[mb] = abase[mb * 64];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+#pragma unroll
+      for (int mb = 0; mb < FB_MB; ++mb) {
+        mfma_inplace<DT>(acc[mb][w][0], af[mb], ocur[w][0]);
+        mfma_inplace<DT>(acc[mb][w][1], af[mb], ocur[w][1]);
+      }
+      // word w of this k-step is done: dequantise word w of the next k-step in place
+      dequant_word(nxt, w, ocur[w][0], ocur[w][1]);
+    }
+  };
+
+  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration
+#pragma unroll 1
+  for (int c0 = 0; c0 < nchunks; c0 += 2) {
+    const int ks0 = 2 * c0;
+    // chunk c0 in buffer 0
+    load_a(c0 + 1);
+    kstep(0, 0, st[1]);
+    issue(st[0], ks0 + 4);
+    kstep(0, 1, st[2]);
+    issue(st[1], ks0 + 5);
+    store_a(1);
+    __syncthreads();
+    // chunk c0+1 in buffer 1
+    load_a(c0 + 2);
+    kstep(1, 0, st[3]);
+    issue(st[2], ks0 + 6);
+    kstep(1, 1, st[0]);
+    issue(st[3], ks0 + 7);
+    store_a(0);
+    __syncthreads();
+  }
+
+  // ------------------------------------------------------------------------------ epilogue
+  // (the inline-asm MFMAs are opaque to the compiler's hazard logic: let the matrix pipe drain before the
+  //  accumulators are read)
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // per wavefront and m-block: accumulators -> private LDS slab [16 rows][RED_RS] -> 8-byte row stores
+  float* slab = (float*)smem + wv * (16 * RED_RS);
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  const int fc4 = (lane & 31) * 4;
+  const int fpos = fc4 + (fc4 >= 64 ? 8 : 0);
+  const int ncol = cp * 128 + fc4;
+  const bool fcol_ok = wave_on && ncol < p.N;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if (fcol_ok) {
+    const int base = ncol & ~31, cl = ncol & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  }
+#pragma unroll
+  for (int mb = 0; mb < FB_MB; ++mb) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) slab[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r16 = (lane >> 5) + 2 * i;
+      const int grow = row0 + mb * 16 + r16;
+      f32x4 v = *(const f32x4*)(slab + r16 * RED_RS + fpos);
+      if (fcol_ok && grow < p.M) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+        u32x2 o;
+        if constexpr (DT == DT_F16)
+          o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+        else
+          o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+        *(u32x2*)((uint16_t*)p.C + (int64_t)grow * p.N + ncol) = o;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+typedef void (*fat_fn)(const KParams);
+
+template <int DT>
+static fat_fn pick_fat2(bool zp, bool channel) {
+  if (zp) return channel ? fat_kernel<DT, true, true> : fat_kernel<DT, true, false>;
+  return channel ? fat_kernel<DT, false, true> : fat_kernel<DT, false, false>;
+}
+
+int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
+  const bool zp = a->b_zeros != nullptr;
+  fat_fn fn = a->dtype == DT_F16 ? pick_fat2<DT_F16>(zp, pl.gm == GM_CHANNEL) : pick_fat2<DT_BF16>(zp, pl.gm == GM_CHANNEL);
+  KParams p = make_kparams(a, pl);
+  const int64_t grid = (int64_t)pl.tiles;
+  if (grid <= 0) return 0;
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), FB_SMEM, stream, p);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace w4a16
