@@ -152,6 +152,47 @@ __device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const Col
   }
 }
 
+// byte N of x as float (v_cvt_f32_ubyteN; the compiler only finds the byte-0 form on its own)
+template <int N>
+__device__ __forceinline__ float ubyte_f32(uint32_t x) {
+  float f;
+  if constexpr (N == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(x));
+  if constexpr (N == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(x));
+  if constexpr (N == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(x));
+  if constexpr (N == 3) asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(x));
+  return f;
+}
+
+// One register (J = 0..7) of what dequant_pair produces: J < 4 -> o0[J], else o1[J - 4].  Lets a caller spread
+// the dequantisation of a Marlin word pair between MFMAs a few instructions at a time.
+template <int DT, bool UNIT_SCALE, int J>
+__device__ __forceinline__ uint32_t dequant_piece(uint32_t xa, uint32_t xb, const ColConst<DT>& cc) {
+  constexpr int HF = J >> 2, Q = J & 3;
+  const uint32_t x = (Q < 2) ? xa : xb;
+  if constexpr (DT == DT_F16) {
+    uint32_t EX = 0x64006400u;
+    asm("" : "+v"(EX));
+    const uint32_t y = HF ? (x >> 8) : x;
+    const f16x2 s = as_h2(cc.s);
+    const f16x2 sc = HF ? f16x2{s.y, s.y} : f16x2{s.x, s.x};
+    f16x2 v;
+    if constexpr ((Q & 1) == 0) {
+      const f16x2 z = as_h2(cc.zl);
+      v = as_h2((y & 0x000f000fu) | EX) - (HF ? f16x2{z.y, z.y} : f16x2{z.x, z.x});
+    } else {
+      const f16x2 z = as_h2(cc.zh);
+      const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+      v = as_h2((y & 0x00f000f0u) | EX) * sixteenth - (HF ? f16x2{z.y, z.y} : f16x2{z.x, z.x});
+    }
+    return as_u32(UNIT_SCALE ? v : v * sc);
+  } else {
+    // nibbles 2*HF + (Q&1) and that + 4: both sit in byte HF / HF + 2 of the even- or odd-nibble word
+    const uint32_t m = ((Q & 1) ? (x >> 4) : x) & 0x0f0f0f0fu;
+    const float sf = HF ? cc.s1 : cc.s0, cf = HF ? cc.c1 : cc.c0;
+    return pack_bf16(__builtin_fmaf(ubyte_f32<HF>(m), sf, cf), __builtin_fmaf(ubyte_f32<HF + 2>(m), sf, cf));
+  }
+}
+
 // "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
 // of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
 // high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the

@@ -15,6 +15,8 @@
 // word-major (16 per Marlin word), and as soon as a word's operands are dead the next k-step's word is
 // dequantised into the same registers.
 // Requirements (host-checked; otherwise the skinny kernel runs): dense op, K % 128 == 0, no per-row g_idx.
+#include <type_traits>
+
 #include "gemm_kernels.h"
 
 namespace w4a16 {
@@ -110,14 +112,13 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
   };
-  auto dequant_word = [&](const Stage& s, int w, u32x4& o0, u32x4& o1) {
+  auto col_const = [&](const Stage& s, int w) {
     uint32_t z0 = 8, z1 = 8;
     if (ZP) {
       z0 = (s.zq >> (4 * w)) & 0xf;
       z1 = (s.zq >> (4 * w + 16)) & 0xf;
     }
-    const ColConst<DT> cc = make_col_const<DT, UNIT>(CHANNEL ? 0u : s.sc[w], z0, z1);
-    dequant_pair<DT, UNIT>(s.b0[w], s.b1[w], cc, o0, o1);
+    return make_col_const<DT, UNIT>(CHANNEL ? 0u : s.sc[w], z0, z1);
   };
 
   f32x4 acc[FB_MB][4][2];
@@ -137,28 +138,56 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
 #pragma unroll
   for (int j = 0; j < FB_D; ++j) issue(st[j], j);
   store_a(0);
-  u32x4 ocur[4][2];
+  // B operands of the current and of the next k-step (the roles swap every k-step)
+  u32x4 ob[2][4][2];
 #pragma unroll
-  for (int w = 0; w < 4; ++w) dequant_word(st[0], w, ocur[w][0], ocur[w][1]);
+  for (int w = 0; w < 4; ++w) {
+    const ColConst<DT> cc = col_const(st[0], w);
+    dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], cc, ob[0][w][0], ob[0][w][1]);
+  }
   __syncthreads();
 
-  // One k-step: 64 MFMAs on `ocur`, interleaved with the dequantisation of the next k-step's words.
-  auto kstep = [&](int buf, int kk, const Stage& nxt) {
+  // One k-step: 64 MFMAs on ob[CUR].  The matrix pipe takes 16 cycles per MFMA, so between every two MFMAs
+  // one register of the next k-step's operands (3-5 VALU instructions) is dequantised into ob[CUR ^ 1]; the
+  // scheduling barriers keep the compiler from regrouping that into MFMA-only and VALU-only blocks, which would
+  // leave the matrix pipe idle during the VALU blocks.
+  auto kstep = [&](auto cur_tag, int buf, int kk, const Stage& nxt) {
+    constexpr int CUR = decltype(cur_tag)::value;
     const u32x4* abase = (const u32x4*)(lds + buf * (FB_ABUF / 4)) + (kk * FB_MB) * 64 + lane;
     u32x4 af[FB_MB];
 #pragma unroll
     for (int mb = 0; mb < FB_MB; ++mb) af[mb] = abase[mb * 64];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-#pragma unroll
-      for (int mb = 0; mb < FB_MB; ++mb) {
-        mfma_inplace<DT>(acc[mb][w][0], af[mb], ocur[w][0]);
-        mfma_inplace<DT>(acc[mb][w][1], af[mb], ocur[w][1]);
-      }
-      // word w of this k-step is done: dequantise word w of the next k-step in place
-      dequant_word(nxt, w, ocur[w][0], ocur[w][1]);
-    }
+    auto word = [&](auto w_tag) {
+      constexpr int w = decltype(w_tag)::value;
+      const ColConst<DT> cc = col_const(nxt, w);
+      const uint32_t xa = nxt.b0[w], xb = nxt.b1[w];
+      auto step = [&](auto j_tag) {
+        constexpr int J = decltype(j_tag)::value;
+        mfma_inplace<DT>(acc[J][w][0], af[J], ob[CUR][w][0]);
+        mfma_inplace<DT>(acc[J][w][1], af[J], ob[CUR][w][1]);
+        const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        if constexpr (J < 4)
+          ob[CUR ^ 1][w][0][J] = r;
+        else
+          ob[CUR ^ 1][w][1][J - 4] = r;
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      step(std::integral_constant<int, 0>{});
+      step(std::integral_constant<int, 1>{});
+      step(std::integral_constant<int, 2>{});
+      step(std::integral_constant<int, 3>{});
+      step(std::integral_constant<int, 4>{});
+      step(std::integral_constant<int, 5>{});
+      step(std::integral_constant<int, 6>{});
+      step(std::integral_constant<int, 7>{});
+    };
+    word(std::integral_constant<int, 0>{});
+    word(std::integral_constant<int, 1>{});
+    word(std::integral_constant<int, 2>{});
+    word(std::integral_constant<int, 3>{});
   };
+  const std::integral_constant<int, 0> even{};
+  const std::integral_constant<int, 1> odd{};
 
   // ---- main loop: two chunks (four k-steps = the weight ring) per iteration
 #pragma unroll 1
@@ -166,17 +195,17 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     const int ks0 = 2 * c0;
     // chunk c0 in buffer 0
     load_a(c0 + 1);
-    kstep(0, 0, st[1]);
+    kstep(even, 0, 0, st[1]);
     issue(st[0], ks0 + 4);
-    kstep(0, 1, st[2]);
+    kstep(odd, 0, 1, st[2]);
     issue(st[1], ks0 + 5);
     store_a(1);
     __syncthreads();
     // chunk c0+1 in buffer 1
     load_a(c0 + 2);
-    kstep(1, 0, st[3]);
+    kstep(even, 1, 0, st[3]);
     issue(st[2], ks0 + 6);
-    kstep(1, 1, st[0]);
+    kstep(odd, 1, 1, st[0]);
     issue(st[3], ks0 + 7);
     store_a(0);
     __syncthreads();
