@@ -1,0 +1,203 @@
+"""MoE glue and the fused-MoE W4A16 path on the GPU against the CPU oracle (reference tests:
+tests/kernels/moe/test_moe.py:667-744, test_moe_align_block_size.py, test_moe.py:889)."""
+import pytest
+import torch
+
+from helpers import make_layer, tol_for
+from oracle import gemm_ref as gr
+from oracle import moe_ref as mr
+
+pytestmark = pytest.mark.gpu
+
+
+def rand_topk(m, topk, e, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+
+
+# ------------------------------------------------------------------------------ align / sum / silu
+def test_align_docstring_example(dev):
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32, device=dev)
+    s, x, t = moe_align_block_size(ids, 4, 5)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert int(t) == 16 and x[:4].tolist() == [1, 2, 3, 4]
+
+
+@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 8, 8), (16, 2, 8, 16), (123, 3, 12, 32), (666, 2, 4, 64),
+                                         (4096, 2, 8, 64), (1000, 6, 256, 16), (3, 8, 1024, 8)])
+@pytest.mark.parametrize("pad", [False, True])
+def test_align_equals_oracle(dev, m, topk, e, bs, pad):
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    ids = rand_topk(m, topk, e, seed=m + e)
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e, pad_sorted_ids=pad)
+    ws, wx, wt = mr.moe_align_block_size(ids, bs, e, pad_sorted_ids=pad)
+    assert torch.equal(t.cpu(), wt)
+    assert torch.equal(s.cpu(), ws)
+    assert torch.equal(x.cpu(), wx)
+
+
+def test_align_expert_map(dev):
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    ids = rand_topk(50, 2, 8, seed=7)
+    emap = torch.tensor([-1, 0, -1, 1, -1, 2, -1, 3], dtype=torch.int32)
+    s, x, t = moe_align_block_size(ids.to(dev), 16, 8, expert_map=emap.to(dev))
+    ws, wx, wt = mr.moe_align_block_size(ids, 16, 8, expert_map=emap)
+    nb = int(wt) // 16
+    assert torch.equal(t.cpu(), wt) and torch.equal(s.cpu(), ws) and torch.equal(x.cpu()[:nb], wx[:nb])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,topk,d", [(1, 2, 64), (37, 3, 4096), (512, 2, 1024)])
+def test_moe_sum(dev, dtype, m, topk, d):
+    import vllm_amd.ops as ops
+    x = torch.randn(m, topk, d, generator=torch.Generator().manual_seed(0)).to(dtype)
+    out = torch.empty(m, d, dtype=dtype, device=dev)
+    ops.moe_sum(x.to(dev), out)
+    want = x.float().sum(dim=1).to(dtype)                      # fp32 accumulate, one rounding
+    assert torch.equal(out.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,d", [(1, 64), (33, 14336), (256, 1024)])
+def test_silu_and_mul(dev, dtype, m, d):
+    import vllm_amd.ops as ops
+    x = torch.randn(m, 2 * d, generator=torch.Generator().manual_seed(1)).to(dtype)
+    out = torch.empty(m, d, dtype=dtype, device=dev)
+    ops.silu_and_mul(out, x.to(dev))
+    xf = x[:, :d].float()
+    want = ((xf / (1 + torch.exp(-xf))).to(dtype) * x[:, d:]).float()   # SiLU in fp32 -> T, then a T multiply
+    got = out.cpu().float()
+    # exp differs in the last ulp between devices: allow one rounding step of the result type
+    eps = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    assert ((got - want).abs() <= eps * want.abs() + 1e-6).all()
+    assert torch.allclose(got, mr.silu_and_mul(x.float()), rtol=4 * eps, atol=1e-3)
+
+
+# ------------------------------------------------------------------------------------- MoE GEMM
+def make_experts(e, k, n, group, dtype, has_zp, act_order, seed):
+    layers = [make_layer(k, n, group, dtype, has_zp=has_zp, act_order=act_order, seed=seed + i, w_std=0.1) for i in range(e)]
+    st = lambda name: torch.stack([getattr(l, name) for l in layers])
+    return layers, st("marlin_q"), st("marlin_s"), st("marlin_zp"), st("g_idx_sorted"), st("sort_indices")
+
+
+@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 4, 8), (33, 2, 8, 16), (123, 3, 4, 32), (200, 2, 4, 48), (333, 2, 4, 64)])
+@pytest.mark.parametrize("variant", ["gptq_f16_g128", "gptq_bf16_chan", "awq_bf16_g128", "gptq_f16_g32_act"])
+@pytest.mark.parametrize("mul", [False, True])
+def test_moe_gemm_equals_oracle(dev, m, topk, e, bs, variant, mul):
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    dtype = torch.bfloat16 if "bf16" in variant else torch.float16
+    group = -1 if "chan" in variant else 32 if "g32" in variant else 128
+    has_zp, act = variant.startswith("awq"), variant.endswith("act")
+    k, n = 256, 192
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, group, dtype, has_zp, act, seed=10)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).to(dtype)
+    ids = rand_topk(m, topk, e, seed=6)
+    tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7))
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e)
+    ws = marlin_make_workspace_new(dev, 4)
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), None, mq.to(dev), None, ms.to(dev), None, mz.to(dev), gi.to(dev), perm.to(dev), ws, s, x, t,
+        tw.to(dev), moe_block_size=bs, top_k=topk, mul_topk_weights=mul, is_ep=False,
+        b_q_type=scalar_types.uint4 if has_zp else scalar_types.uint4b8, size_m=m, size_n=n, size_k=k,
+        is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
+    assert out.shape == (m * topk, n)
+    w_dense = torch.stack([l.w_ref for l in layers])
+    ref = mr.moe_gemm_ref(a, w_dense, s.cpu(), x.cpu(), t.cpu(), tw, bs, topk, mul, m)
+    mtr = gr.error_metrics(out, ref)
+    assert mtr["max_rel"] <= tol_for(dtype) and mtr["mean_rel"] < 0.04, mtr
+    assert int(ws.abs().sum()) == 0
+
+
+def test_moe_gemm_skips_foreign_experts_and_bias(dev):
+    """expert_ids = -1 blocks are left untouched (expert parallelism); per-expert bias is added."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new, marlin_permute_bias
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    m, topk, e, bs, k, n = 40, 2, 4, 16, 256, 128
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, 128, torch.float16, False, False, seed=30)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(8)).half()
+    ids = rand_topk(m, topk, e, seed=9)
+    emap = torch.tensor([0, -1, 1, -1], dtype=torch.int32)
+    bias = torch.randn(e, n, generator=torch.Generator().manual_seed(10)).half()
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e, expert_map=emap.to(dev))
+    c = torch.full((m * topk, n), 7.0, dtype=torch.float16, device=dev)
+    # local experts 0, 1 hold global experts 0, 2
+    local = [0, 2]
+    pb = torch.stack([marlin_permute_bias(bias[g]) for g in local])
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), c, mq[local].to(dev), pb.to(dev), ms[local].to(dev), None, mz[local].to(dev), gi[local].to(dev),
+        perm[local].to(dev), marlin_make_workspace_new(dev, 4), s, x, t, torch.ones(m, topk, device=dev),
+        moe_block_size=bs, top_k=topk, mul_topk_weights=False, is_ep=True, b_q_type=scalar_types.uint4b8,
+        size_m=m, size_n=n, size_k=k, is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
+    out = out.cpu().float()
+    flat = ids.flatten()
+    for i in range(m * topk):
+        g = int(flat[i])
+        if int(emap[g]) < 0:
+            assert (out[i] == 7.0).all()
+        else:
+            want = a[i // topk].float() @ layers[g].w_ref.float() + bias[g].float()
+            assert float((out[i] - want).abs().max() / want.abs().max()) <= 2e-2
+
+
+# ----------------------------------------------------------------------------------- fused MoE
+@pytest.mark.parametrize("m", [1, 33, 123, 666])
+@pytest.mark.parametrize("e,topk", [(4, 2), (12, 3)])
+@pytest.mark.parametrize("variant", ["gptq_f16_g128", "awq_bf16_g128", "gptq_bf16_chan"])
+def test_fused_marlin_moe_vs_torch_moe(dev, m, e, topk, variant):
+    """The reference's gate: atol 5e-2, rtol 0 against torch_moe on the dequantised weights."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    dtype = torch.bfloat16 if "bf16" in variant else torch.float16
+    group = -1 if "chan" in variant else 128
+    has_zp = variant.startswith("awq")
+    k, inter = 256, 128
+    l1, q1, s1, z1, _, _ = make_experts(e, k, 2 * inter, group, dtype, has_zp, False, seed=100)
+    l2, q2, s2, z2, _, _ = make_experts(e, inter, k, group, dtype, has_zp, False, seed=200)
+    g = torch.Generator().manual_seed(11)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    score = torch.randn(m, e, generator=g).to(dtype)
+    p = torch.softmax(score.float(), dim=-1)
+    tw, ti = torch.topk(p, topk)
+    from helpers import Layer  # noqa: F401
+    out = fused_marlin_moe(
+        a.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), score.to(dev), tw.to(dev),
+        ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e,
+        w1_zeros=z1.to(dev) if has_zp else None, w2_zeros=z2.to(dev) if has_zp else None)
+    w1 = torch.stack([l.w_ref.t() for l in l1])            # [E, 2I, K] as nn.Linear weights
+    w2 = torch.stack([l.w_ref.t() for l in l2])            # [E, K, I]
+    ref = mr.torch_experts(a, w1, w2, tw, ti)
+    assert out.shape == (m, k)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
+
+
+def test_fused_marlin_moe_mixtral_shape(dev):
+    """Mixtral-8x7B expert shapes (hidden 4096, intermediate 14336, top-2) at T = 16; two experts instead of
+    eight, so that quantising them with the CPU oracle stays within seconds."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    e, topk, k, inter, m = 2, 2, 4096, 14336, 16
+    dtype = torch.float16
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=300)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 128, dtype, False, False, seed=400)
+    g = torch.Generator().manual_seed(12)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    score = torch.randn(m, e, generator=g)
+    tw, ti = torch.topk(torch.softmax(score, dim=-1), topk)
+    tw = tw / tw.sum(dim=-1, keepdim=True)
+    out = fused_marlin_moe(a.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), score.to(dev),
+                           tw.to(dev), ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e)
+    # oracle on the GPU-free path would need 8 x (4096x28672 + 14336x4096) fp32 matmuls: do the experts hit only
+    w1 = {int(x): l1[int(x)].w_ref.float() for x in ti.unique()}
+    w2 = {int(x): l2[int(x)].w_ref.float() for x in ti.unique()}
+    ref = torch.zeros(m, k)
+    for t in range(m):
+        for j in range(topk):
+            ex = int(ti[t, j])
+            h = (a[t].float() @ w1[ex]).to(dtype)
+            act = (torch.nn.functional.silu(h[:inter].float()).to(dtype) * h[inter:])
+            ref[t] += float(tw[t, j]) * (act.float() @ w2[ex]).to(dtype).float()
+    torch.testing.assert_close(out.cpu().float(), ref, atol=5e-2, rtol=0)

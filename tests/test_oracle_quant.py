@@ -1,0 +1,163 @@
+"""Pins the oracle's quantizers, checkpoint packers, type ids and dequantisation (CPU only)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm_ref as gr
+from oracle import marlin_layout as ml
+from oracle import quant_utils as qu
+from oracle import scalar_types as st
+
+
+def u32(t):
+    return t.numpy().view(np.uint32)
+
+
+# ---------------------------------------------------------------------------------- type ids
+def test_type_ids_literal():
+    # mantissa << 8 | bias << 17 | nan_repr(IEEE = 1) << 50
+    assert st.uint4.id == (4 << 8) | (1 << 50) == 1125899906843648
+    assert st.uint4b8.id == (4 << 8) | (8 << 17) | (1 << 50) == 1125899907892224
+    assert st.uint8b128.id == (8 << 8) | (128 << 17) | (1 << 50) == 1125899923621888
+    assert (st.uint4b8.min(), st.uint4b8.max()) == (-8, 7)
+    assert (st.uint4.min(), st.uint4.max()) == (0, 15)
+
+
+# ----------------------------------------------------------------------------------- packers
+def test_pack_rows_literal_and_roundtrip():
+    q = torch.arange(8, dtype=torch.int32).view(8, 1)            # rows 0..7 -> nibble i = i
+    assert int(u32(qu.pack_rows(q, 4))[0, 0]) == 0x76543210
+    q = torch.tensor([[15]] * 8, dtype=torch.int32)
+    assert int(qu.pack_rows(q, 4)[0, 0]) == -1                   # 0xffffffff as int32
+    r = torch.randint(0, 16, (64, 24), generator=torch.Generator().manual_seed(0), dtype=torch.int32)
+    assert torch.equal(qu.unpack_rows(qu.pack_rows(r, 4), 4), r)
+    assert qu.gptq_pack(r).shape == (8, 24)
+
+
+def test_pack_cols_literal_and_roundtrip():
+    q = torch.arange(8, dtype=torch.int32).view(1, 8)
+    assert int(u32(qu.pack_cols(q, 4))[0, 0]) == 0x76543210
+    r = torch.randint(0, 16, (5, 64), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    assert torch.equal(qu.unpack_cols(qu.pack_cols(r, 4), 4), r)
+
+
+def test_awq_pack_literal_and_roundtrip():
+    # nibble t of the word holds column (0,2,4,6,1,3,5,7)[t]
+    q = torch.arange(8, dtype=torch.int32).view(1, 8)
+    assert int(u32(qu.awq_pack(q))[0, 0]) == 0x75316420
+    r = torch.randint(0, 16, (7, 128), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    assert torch.equal(qu.awq_unpack(qu.awq_pack(r)), r)
+    # brute force
+    p = u32(qu.awq_pack(r))
+    for c in range(16):
+        word = 0
+        for t, o in enumerate((0, 2, 4, 6, 1, 3, 5, 7)):
+            word |= int(r[3, 8 * c + o]) << (4 * t)
+        assert int(p[3, c]) == word
+
+
+# -------------------------------------------------------------------------------- quantizers
+def test_symmetric_rule_hand_built_groups():
+    """uint4b8: s = max(|max/7|, |min/-8|); stored value = round(w/s) + 8."""
+    w = torch.zeros(8, 2, dtype=torch.float32)
+    w[:, 0] = torch.tensor([7.0, -3.5, 0, 1, 2, 3, -1, -2])      # max 7 -> s = 1 ; -3.5 -> round-half-even -4
+    w[:, 1] = torch.tensor([-16.0, 14, 0, 2, 4, 6, -2, -4])      # |min|/8 = 2 = max/7
+    w_ref, q, s, zp = qu.quantize_weights(w, st.uint4b8, 8)
+    assert zp is None
+    assert s.tolist() == [[1.0, 2.0]]
+    assert q[:, 0].tolist() == [15, 4, 8, 9, 10, 11, 7, 6]
+    assert q[:, 1].tolist() == [0, 15, 8, 9, 10, 11, 7, 6]
+    assert torch.equal(w_ref, (q - 8).float() * s.repeat_interleave(8, 0))
+
+
+def test_zero_point_rule_hand_built_group():
+    """uint4 + zp: s = (max-min)/15, zp = round(|min/s|), q = clamp(round(w/s) + zp, 0, 15)."""
+    w = torch.tensor([[-5.0], [10.0], [0.0], [1.0], [2.4], [-1.0], [7.0], [9.6]])
+    w_ref, q, s, zp = qu.quantize_weights(w, st.uint4, 8, zero_points=True)
+    assert s.tolist() == [[1.0]] and zp.tolist() == [[5]]
+    assert q[:, 0].tolist() == [0, 15, 5, 6, 7, 4, 12, 15]
+    assert torch.equal(w_ref[:, 0], (q[:, 0] - 5).float())
+
+
+def test_benchmark_rules():
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(256, 16, generator=g) * 0.02).half()
+    w_ref, q, s = qu.quantize_absmax7(w, 128)
+    wg = w.float().view(2, 128, 16)
+    assert torch.equal(s, (wg.abs().amax(1) / 7).half())
+    assert q.min() >= 1 and q.max() <= 15                       # absmax/7 never reaches -8
+    assert torch.equal(w_ref, ((q - 8).half().view(2, 128, 16) * s.view(2, 1, 16)).view(256, 16))
+    w_ref, q, s, zp = qu.quantize_minmax_zp(w.bfloat16(), 128)
+    assert q.min() >= 0 and q.max() <= 15 and zp.min() >= 0 and zp.max() <= 15
+    assert torch.equal(w_ref, ((q.view(2, 128, 16) - zp.view(2, 1, 16)).bfloat16() * s.view(2, 1, 16)).view(256, 16))
+
+
+@pytest.mark.parametrize("group", [-1, 32, 128])
+def test_channelwise_and_group_shapes(group):
+    w = torch.randn(256, 64, generator=torch.Generator().manual_seed(3)).half()
+    w_ref, q, s, _ = qu.quantize_weights(w, st.uint4b8, group)
+    assert s.shape == (1 if group == -1 else 256 // group, 64)
+    assert q.min() >= 0 and q.max() <= 15
+    # reconstruction error bounded by half a step per element
+    gs = 256 if group == -1 else group
+    step = s.float().repeat_interleave(gs, 0)
+    assert ((w.float() - w_ref.float()).abs() <= 0.5 * step * 1.01 + 1e-3).all()
+
+
+def test_act_order_identities():
+    g = torch.Generator().manual_seed(4)
+    w = torch.randn(256, 64, generator=g).half()
+    perm = torch.randperm(256, generator=g)
+    w_ref, q, s, g_idx, rp = qu.gptq_quantize_weights(w, st.uint4b8, 64, True, perm)
+    w0, q0, s0, _ = qu.quantize_weights(w, st.uint4b8, 64)
+    assert torch.equal(rp, perm) and torch.equal(s, s0)
+    assert torch.equal(q, q0[perm]) and torch.equal(w_ref, w0[perm])
+    assert torch.equal(g_idx.long(), perm // 64)
+    qs, gs, order = qu.sort_weights(q, g_idx)
+    assert (gs[1:] >= gs[:-1]).all()
+    assert torch.equal(qs, q[order.long()])
+    assert torch.equal(torch.bincount(gs.long()), torch.full((4,), 64))
+
+
+# -------------------------------------------------------------------- dequantisation identity
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 32, 128])
+@pytest.mark.parametrize("mode", ["gptq", "gptq_act_order", "awq"])
+def test_dequant_reproduces_quantizer_w_ref(dtype, group, mode):
+    k, n = 256, 128
+    if mode == "gptq_act_order" and group == -1:
+        pytest.skip("act-order needs groups")
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(k, n, generator=g).to(dtype)
+    gs = k if group == -1 else group
+    if mode == "awq":
+        w_ref, q, s, zp = qu.quantize_weights(w, st.uint4, group, zero_points=True)
+        mq = ml.awq_marlin_repack(qu.awq_pack(q), k, n)
+        mz = ml.awq_to_marlin_zero_points(qu.awq_pack(zp), zp.shape[0], n)
+        ms = ml.marlin_permute_scales(s, k, n, gs)
+        assert torch.equal(gr.dequant_marlin(mq, ms, mz, None, k, n, False, dtype), w_ref)
+        assert torch.equal(gr.dequant_checkpoint(qu.awq_pack(q), s, qu.awq_pack(zp), None, "awq", dtype), w_ref)
+        return
+    act = mode == "gptq_act_order"
+    w_ref, q, s, g_idx, _ = qu.gptq_quantize_weights(w, st.uint4b8, group, act, torch.randperm(k, generator=g) if act else None)
+    ms = ml.marlin_permute_scales(s, k, n, gs)
+    if act:
+        _, g_sorted, order = qu.sort_weights(q, g_idx)
+        mq = ml.gptq_marlin_repack(qu.gptq_pack(q), order, k, n)
+        w_sorted = gr.dequant_marlin(mq, ms, None, g_sorted, k, n, True, dtype)
+        assert torch.equal(w_sorted, w_ref[order.long()])
+        assert torch.equal(gr.dequant_checkpoint(qu.gptq_pack(q), s, None, g_idx, "gptq", dtype), w_ref)
+    else:
+        mq = ml.gptq_marlin_repack(qu.gptq_pack(q), None, k, n)
+        assert torch.equal(gr.dequant_marlin(mq, ms, None, None, k, n, True, dtype), w_ref)
+        assert torch.equal(gr.dequant_checkpoint(qu.gptq_pack(q), s, None, None, "gptq", dtype), w_ref)
+
+
+def test_gemm_ref_is_fp32_matmul_plus_bias():
+    a = torch.tensor([[1.0, 2.0], [0.5, -1.0]]).half()
+    w = torch.tensor([[2.0, 0.0], [1.0, 4.0]]).half()
+    out = gr.gemm_ref(a, w, torch.tensor([1.0, -1.0]).half())
+    assert out.dtype == torch.float32
+    assert out.tolist() == [[5.0, 7.0], [1.0, -5.0]]
+    m = gr.error_metrics(out + torch.tensor([[0.0, 0.7], [0.0, 0.0]]), out)
+    assert abs(m["max_rel"] - 0.1) < 1e-6 and abs(m["mean_rel"] - 0.7 / 18.0) < 1e-6

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     if (p.moe) {
       if (r < p.moe_bs) {
         const int id = p.sorted_ids[mt * p.moe_bs + r];
-        if (id < p.c_rows) {
+        if ((unsigned)id < (unsigned)p.c_rows) {
           src = id / p.top_k;
           dst = id;
         }
@@ -99,6 +99,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   {
     int src0, dst0;
     tile_row_ids(0, src0, dst0);
+    if (src0 < 0) src0 = 0;  // a block whose first slot is padding still reads inside A
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       int src, dst;
