@@ -159,6 +159,96 @@ def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=4
             "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS, "max_rel_err": err}
 
 
+def make_gptq_actorder_layer(ops, k, n, dtype, dev, seed):
+    """GPTQ desc_act layer: rows arrive in a seeded random order, g_idx[i] = group of arriving row i
+    (as the reference's permute_rows, quant_utils.py:346-373); weights are repacked in group-sorted order."""
+    base = make_gptq_layer(ops, k, n, dtype, dev, seed)
+    g = torch.Generator(device="cpu").manual_seed(seed + 7)
+    perm = torch.randperm(k, generator=g).to(dev)
+    g_idx = (perm // GROUP).to(torch.int32)
+    order = torch.argsort(g_idx, stable=True).to(torch.int32)
+    packed_arrival = _pack_rows_gpu(_unpack_rows_gpu(base["packed"])[perm])
+    mq = ops.gptq_marlin_repack(packed_arrival, order, k, n, 4)
+    return {**base, "q": mq, "g_idx": g_idx[order.long()].contiguous(), "perm": order, "w_deq": base["w_deq"][perm]}
+
+
+def _unpack_rows_gpu(p):  # GPTQ int32 [K/8, N] -> [K, N]
+    sh = (torch.arange(8, device=p.device, dtype=torch.int64) * 4).view(1, 8, 1)
+    return (((p.to(torch.int64) & 0xFFFFFFFF).unsqueeze(1) >> sh) & 0xF).reshape(-1, p.shape[1]).to(torch.int32)
+
+
+def bench_act_order(ops, wtype, dev, workspace):
+    """BASELINE config 4: down_proj (K=14336, N=4096), g128, desc_act, fp16, M in {1, 16, 512}."""
+    k, n = LAYERS["down"]
+    base = make_gptq_actorder_layer(ops, k, n, torch.float16, dev, 21)
+    ncopy = copies_needed(base["q"].numel() * 4)
+    copies = [base] + [clone_weights(base, 300 + i) for i in range(ncopy - 1)]
+    out = {}
+    for m in (1, 16, 512):
+        a = torch.randn(m, k, generator=torch.Generator().manual_seed(4)).half().to(dev)
+        call = lambda l: ops.gptq_marlin_gemm(a, None, l["q"], None, l["s"], None, l["zp"], base["g_idx"], base["perm"],
+                                              workspace, wtype, m, n, k, True, False, True, False)
+        res = call(base)
+        ref = a.float() @ base["w_deq"].float()
+        err = float((res.float() - ref).abs().max() / ref.abs().max())
+        fns = [(lambda c=copies[i % ncopy]: call(c)) for i in range(max(16, ncopy))]
+        sec = time_graph(fns, reps=3, warmup=1) / len(fns)
+        by, fl = algorithmic_bytes(m, k, n, act_order=True), 2.0 * m * n * k
+        out[f"down_M{m}"] = {"m": m, "k": k, "n": n, "us": sec * 1e6, "GBps": by / sec / 1e9, "TFLOPs": fl / sec / 1e12,
+                             "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS, "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS,
+                             "max_rel_err": err}
+        print(f"[detail] act-order down M={m}: {sec * 1e6:.2f} us, {by / sec / 1e9:.0f} GB/s = "
+              f"{100 * by / sec / 1e9 / HBM_PEAK_GBPS:.1f}% HBM, {fl / sec / 1e12:.1f} TFLOP/s, err {err:.1e}",
+              file=sys.stderr, flush=True)
+    return out
+
+
+def bench_moe(ops, wtype, dev):
+    """BASELINE config 5: Mixtral-8x7B fused MoE (8 experts, hidden 4096, intermediate 14336, top-2), uint4b8 g128
+    fp16, T in {16, 512, 4096}; one call = align + GEMM1 + SiLU-and-mul + GEMM2 + top-k sum."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    e, hid, inter, topk = 8, 4096, 14336, 2
+    w13 = [make_gptq_layer(ops, hid, 2 * inter, torch.float16, dev, 40 + i) for i in range(e)]
+    w2 = [make_gptq_layer(ops, inter, hid, torch.float16, dev, 60 + i) for i in range(e)]
+    q1, s1 = torch.stack([l["q"] for l in w13]), torch.stack([l["s"] for l in w13])
+    q2, s2 = torch.stack([l["q"] for l in w2]), torch.stack([l["s"] for l in w2])
+    deq13 = [l["w_deq"] for l in w13]
+    deq2 = [l["w_deq"] for l in w2]
+    del w13, w2
+    per_expert = (hid * 2 * inter + inter * hid) // 2 + ((hid // GROUP) * 2 * inter + (inter // GROUP) * hid) * 2
+    out = {}
+    for t in (16, 512, 4096):
+        g = torch.Generator().manual_seed(5)
+        x = (torch.randn(t, hid, generator=g)).half().to(dev)
+        logits = torch.randn(t, e, generator=g).to(dev)
+        tw, ti = torch.topk(torch.softmax(logits.float(), dim=-1), topk)
+        tw = (tw / tw.sum(dim=-1, keepdim=True)).contiguous()
+        ti = ti.to(torch.int32).contiguous()
+        call = lambda: fused_marlin_moe(x, q1, q2, None, None, s1, s2, logits, tw, ti, quant_type_id=wtype.id,
+                                        global_num_experts=e)
+        res = call()
+        # check the first 4 tokens against dequantised fp32 matmuls on the GPU
+        ref = torch.zeros(4, hid, device=dev)
+        for r in range(min(4, t)):
+            for j in range(topk):
+                ex = int(ti[r, j])
+                h = (x[r].float() @ deq13[ex].float()).half()
+                act = (torch.nn.functional.silu(h[:inter].float()).half() * h[inter:])
+                ref[r] += float(tw[r, j]) * (act.float() @ deq2[ex].float()).half().float()
+        err = float((res[:4].float() - ref[:min(4, t)]).abs().max() / ref.abs().max())
+        sec = time_graph([call] * 4, reps=3, warmup=1) / 4
+        hit = int(ti.unique().numel())
+        by = hit * per_expert + t * hid * 2 * 2 + t * topk * (2 * inter + inter + hid) * 2 * 2
+        fl = 2.0 * t * topk * (hid * 2 * inter + inter * hid)
+        out[f"T{t}"] = {"tokens": t, "experts_hit": hit, "us": sec * 1e6, "GBps": by / sec / 1e9, "TFLOPs": fl / sec / 1e12,
+                        "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS, "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS,
+                        "max_rel_err_first4": err}
+        print(f"[detail] mixtral moe T={t}: {sec * 1e6:.1f} us, {by / sec / 1e9:.0f} GB/s = "
+              f"{100 * by / sec / 1e9 / HBM_PEAK_GBPS:.1f}% HBM, {fl / sec / 1e12:.1f} TFLOP/s = "
+              f"{100 * fl / sec / 1e12 / MFMA_PEAK_TFLOPS:.1f}% MFMA, err {err:.1e}", file=sys.stderr, flush=True)
+    return out
+
+
 def cpu_baseline(m, budget_s=12.0):
     """The oracle's CPU path (unpack GPTQ nibbles, (q-8)*s group-broadcast, torch.matmul in fp32) on the
     host cores: whole passes over the four layers at M=`m`, repeated until `budget_s` seconds of CPU work."""
@@ -300,7 +390,7 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_detail:
-        detail = {"decode_fp16_gptq": {}, "prefill_bf16_awq": {}}
+        detail = {"decode_fp16_gptq": {}, "prefill_bf16_awq": {}}  # + act_order_fp16_gptq, mixtral_moe_fp16_gptq
         for name, (k, n) in LAYERS.items():
             for mm in (1, 4, 16, 64, 256):
                 r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_layer(ops, *a), mm, k, n,
@@ -315,6 +405,10 @@ def main():
             detail["prefill_bf16_awq"][f"{name}_M4096"] = r
             print(f"[detail] {name} M=4096 bf16 awq: {r['us']:.1f} us, {r['TFLOPs']:.1f} TFLOP/s = "
                   f"{100 * r['mfma_frac']:.1f}% MFMA peak", file=sys.stderr, flush=True)
+        detail["act_order_fp16_gptq"] = bench_act_order(ops, scalar_types.uint4b8, dev, workspace)
+        torch.cuda.empty_cache()
+        detail["mixtral_moe_fp16_gptq"] = bench_moe(ops, scalar_types.uint4b8, dev)
+        torch.cuda.empty_cache()
         result["detail"] = detail
         if args.table:
             with open(args.table, "w") as f:

@@ -86,7 +86,10 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
 
-  pl.atmp_bytes = 0;
+  // Dense act-order: A's columns are gathered once into a_tmp by permute_cols (as the reference's
+  // permute_cols_kernel, csrc/quantization/gptq_marlin/gptq_marlin.cu:68-120), so the GEMM kernels read A with
+  // plain 128-bit loads.  MoE blocks gather inside the kernel (rows and per-expert column order together).
+  pl.atmp_bytes = (act_order && !moe) ? a->size_m * a->size_k * 2 : 0;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   static const int fat_min_m = env_int("W4A16_FAT_MIN_M", 128);
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
@@ -105,7 +108,6 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = pl.total_ksteps;
     pl.xcd_map = 0;
     pl.ctmp_bytes = 0;
-    if (pl.use_perm) pl.atmp_bytes = a->size_m * a->size_k * 2;
     return 0;
   }
 
@@ -191,18 +193,14 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
   if (pl.ctmp_bytes + pl.atmp_bytes > 0)
     W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed",
                 (long long)(pl.ctmp_bytes + pl.atmp_bytes));
-  if (pl.kind == 2) {
-    w4a16_gemm_args b = *args;
-    if (pl.use_perm) {
-      // act-order in front of the prefill kernel: gather A's columns once (as the reference's permute_cols_kernel,
-      // csrc/quantization/gptq_marlin/gptq_marlin.cu:549-564), then run the plain grouped path on the copy
-      void* a_tmp = (char*)args->c_tmp + ((pl.ctmp_bytes + 255) & ~255LL);
-      if (int rc = w4a16_permute_cols(args->a, args->perm, a_tmp, args->size_m, args->size_k, args->lda, stream)) return rc;
-      b.a = a_tmp;
-      b.lda = args->size_k;
-      pl.use_perm = false;
-    }
-    return launch_fat(&b, pl, (hipStream_t)stream);
+  w4a16_gemm_args b = *args;
+  if (pl.atmp_bytes > 0) {
+    void* a_tmp = (char*)args->c_tmp + ((pl.ctmp_bytes + 255) & ~255LL);
+    if (int rc = w4a16_permute_cols(args->a, args->perm, a_tmp, args->size_m, args->size_k, args->lda, stream)) return rc;
+    b.a = a_tmp;
+    b.lda = args->size_k;
+    pl.use_perm = false;
   }
-  return pl.kind == 1 ? launch_decode(args, pl, (hipStream_t)stream) : launch_skinny(args, pl, (hipStream_t)stream);
+  if (pl.kind == 2) return launch_fat(&b, pl, (hipStream_t)stream);
+  return pl.kind == 1 ? launch_decode(&b, pl, (hipStream_t)stream) : launch_skinny(&b, pl, (hipStream_t)stream);
 }

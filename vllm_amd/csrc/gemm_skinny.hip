@@ -476,7 +476,7 @@ static skinny_fn pick_zp_gm(bool zp, int gm) {
   if (gm == GM_CHANNEL) {
     if constexpr (PERM) return nullptr; else return skinny_kernel<DT, MB, false, GM_CHANNEL, false>;
   }
-  if constexpr (PERM) return skinny_kernel<DT, MB, false, GM_GIDX, true>; else return nullptr;
+  return skinny_kernel<DT, MB, false, GM_GIDX, PERM>;
 }
 
 template <int DT, bool PERM>
