@@ -90,11 +90,12 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // permute_cols_kernel, csrc/quantization/gptq_marlin/gptq_marlin.cu:68-120), so the GEMM kernels read A with
   // plain 128-bit loads.  MoE blocks gather inside the kernel (rows and per-expert column order together).
   pl.atmp_bytes = (act_order && !moe) ? a->size_m * a->size_k * 2 : 0;
+  const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   static const int fat_min_m = env_int("W4A16_FAT_MIN_M", 128);
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
   if (!moe && a->size_m >= fat_min_m && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
-      pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1) {
+      pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
     pl.mb = 8;
@@ -111,48 +112,87 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     return 0;
   }
 
+  // 64-row kernel: MoE blocks of 64 slots, and dense problems with too few rows or tiles for the prefill kernel
+  // but enough 64 x 512 tiles to occupy the chip without splitting K.
+  {
+    const int64_t mid_mtiles = moe ? ceil_div(a->n_sorted, 64) : ceil_div(a->size_m, 64);
+    const int64_t mid_tiles = mid_mtiles * ceil_div(a->size_n, 512);
+    const bool mid_shape = a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+                           (moe ? a->moe_block_size == 64 : (a->size_m > 32 && mid_tiles >= cus / 2));
+    if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
+      W4A16_CHECK(mid_tiles < (1LL << 31) / 64, "too many tiles");
+      pl.kind = 3;
+      pl.tn = 512;
+      pl.mb = 4;
+      pl.bm = 64;
+      pl.mtiles = (int)mid_mtiles;
+      pl.ncp = (int)ceil_div(a->size_n, 512);
+      pl.tiles = (int)mid_tiles;
+      pl.splits = 1;
+      pl.kps = pl.total_ksteps;
+      pl.xcd_map = 0;
+      pl.ctmp_bytes = 0;
+      return 0;
+    }
+  }
+
   // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
-  const bool decode_ok = pl.mb == 1 && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
-                         (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
+  const bool decode_shape = pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
+                            (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
 
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these
-  // kernels: one 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~21 GB/s on a 64-column
-  // strip (instruction-issue bound), the whole chip ~4.7 TB/s; summing K-splits across workgroups adds
-  // ~3 us of dependent device-scope round trips.  Only one such workgroup fits a compute unit, so a grid
-  // larger than the number of compute units runs in rounds.  Each split needs >= 1 stage per wavefront and
-  // one workspace counter per tile.
-  struct Cand { int kind, tn, splits; double t; };
-  Cand best{0, 128, 1, 1e30};
-  const int n_tn = decode_ok ? 2 : 1;
-  for (int ti = 0; ti < n_tn; ++ti) {
-    const int tn = ti == 0 ? 128 : 64;
-    if (forced_tn && tn != forced_tn && decode_ok) continue;
-    const int64_t ncol_tiles = ceil_div(a->size_n, tn);
-    const int64_t tiles = (int64_t)pl.mtiles * ncol_tiles;
-    if (tiles <= 0 || tiles >= (1LL << 31) / 64) continue;
-    const double bytes = (double)tiles * a->size_k * tn / 2.0;
-    const double wg_rate = (tn == 64 ? 21e3 : 33e3) / (pl.mb > 1 ? 1.5 : 1.0);  // bytes per us
-    const double chip_rate = 4.7e6;
-    const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
-    const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
-    for (int sp = 1; sp <= 16; ++sp) {
-      if (sp > max_splits) break;
-      if (sp > 1 && (!a->workspace || tiles > a->workspace_len)) break;
-      if (forced_splits > 0 && sp != (forced_splits < max_splits ? forced_splits : max_splits)) continue;
-      const int64_t wgs = tiles * sp;
-      if (sp > 1 && wgs > cus) break;
-      const int64_t rounds = ceil_div(wgs, cus);
-      double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
-      if (rate > chip_rate) rate = chip_rate;
-      // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
-      const double t_fix = sp > 1 ? 2.8 + sp * (double)(pl.bm * tn * 4) / 20e3 : 0.0;
-      const double t = bytes / rate + t_fix;
-      if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, t};
+  // kernels.  One 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~21 GB/s on a 64-column
+  // strip with 16-row tiles (instruction-issue bound), ~12 / ~9 GB/s with 32- / 64-row tiles (dequantisation
+  // per element); the whole chip ~4.7 TB/s; summing K-splits across workgroups adds ~3 us of dependent
+  // device-scope round trips plus the last workgroup's pass over the partial tiles.  Only one such workgroup
+  // fits a compute unit, so a grid larger than the number of compute units runs in rounds.  Each split needs
+  // >= 1 stage per wavefront and one workspace counter per tile.
+  // Dense problems of up to 128 rows may also run as several 16-row tiles of the decode kernel: the weight strip
+  // is then re-read from L2 by every row tile, but there is no per-element dequantisation and no K split.
+  struct Cand { int kind, tn, splits, mb; double t; };
+  Cand best{0, 128, 1, pl.mb, 1e30};
+  const int natural_mb = pl.mb;
+  for (int mi = 0; mi < 2; ++mi) {
+    const int mb = mi == 0 ? natural_mb : 1;
+    if (mi == 1 && (natural_mb == 1 || moe || a->size_m > 128 || !decode_shape)) continue;
+    const bool decode_ok = mb == 1 && decode_shape;
+    const int64_t mtiles = moe ? pl.mtiles : ceil_div(a->size_m, 16 * mb);
+    const int n_tn = decode_ok ? 2 : 1;
+    for (int ti = 0; ti < n_tn; ++ti) {
+      const int tn = ti == 0 ? 128 : 64;
+      if (forced_tn && tn != forced_tn && decode_ok) continue;
+      const int64_t ncol_tiles = ceil_div(a->size_n, tn);
+      const int64_t tiles = mtiles * ncol_tiles;
+      if (tiles <= 0 || tiles >= (1LL << 31) / 64) continue;
+      const double bytes = (double)tiles * a->size_k * tn / 2.0;
+      const double wg_rate = mb == 1 ? (tn == 64 ? 21e3 : 33e3) : mb == 2 ? 12e3 : 9e3;  // bytes per us
+      const double chip_rate = 4.7e6;
+      const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
+      const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
+      for (int sp = 1; sp <= 16; ++sp) {
+        if (sp > max_splits) break;
+        if (sp > 1 && (!a->workspace || tiles > a->workspace_len)) break;
+        if (forced_splits > 0 && sp != (forced_splits < max_splits ? forced_splits : max_splits)) continue;
+        const int64_t wgs = tiles * sp;
+        if (sp > 1 && wgs > cus) break;
+        const int64_t rounds = ceil_div(wgs, cus);
+        double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
+        if (rate > chip_rate) rate = chip_rate;
+        // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
+        const double t_fix = sp > 1 ? 2.8 + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
+        const double t = bytes / rate + t_fix;
+        if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, mb, t};
+      }
     }
   }
   W4A16_CHECK(best.t < 1e30, "no launch shape for this problem (too many tiles)");
   pl.kind = best.kind;
   pl.tn = best.tn;
+  if (!moe) {
+    pl.mb = best.mb;
+    pl.bm = 16 * pl.mb;
+    pl.mtiles = (int)ceil_div(a->size_m, pl.bm);
+  }
   pl.ncp = (int)ceil_div(a->size_n, pl.tn);
   pl.tiles = pl.mtiles * pl.ncp;
   {
@@ -202,5 +242,6 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
     pl.use_perm = false;
   }
   if (pl.kind == 2) return launch_fat(&b, pl, (hipStream_t)stream);
+  if (pl.kind == 3) return launch_mid(&b, pl, (hipStream_t)stream);
   return pl.kind == 1 ? launch_decode(&b, pl, (hipStream_t)stream) : launch_skinny(&b, pl, (hipStream_t)stream);
 }

@@ -27,18 +27,6 @@ constexpr int FB_D = 4;      // weight k-steps in flight per wavefront
 constexpr int FB_ABUF = 2 * FB_MB * 64 * 16;  // bytes of one A buffer: 2 k-steps x 8 m-blocks x 64 lanes x 16 B
 constexpr int FB_SMEM = (2 * FB_ABUF > 4 * 16 * RED_RS * 4) ? 2 * FB_ABUF : 4 * 16 * RED_RS * 4;
 
-// In-place MFMA on an accumulator pinned to AGPRs.  With 256 accumulators per lane the register allocator
-// otherwise assigns different registers to an MFMA's source and destination accumulator and fills the loop
-// with v_accvgpr moves (more of them than dequantisation instructions).  Source C == destination is the form
-// the matrix pipe forwards without extra wait states; results are only read again after the main loop.
-template <int DT>
-__device__ __forceinline__ void mfma_inplace(f32x4& acc, const u32x4& a, const u32x4& b) {
-  if constexpr (DT == DT_F16)
-    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-  else
-    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-
 template <int DT, bool ZP, bool CHANNEL>
 __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   constexpr bool UNIT = CHANNEL;

@@ -31,6 +31,7 @@ struct KParams {
   const int32_t* ntpp;
   const float* topk_w;
   int moe, moe_bs, top_k, mul_topk;
+  int n_sorted;  // usable length of sorted_ids
   int64_t b_estride, s_estride, z_estride, k_estride, n_estride;  // per-expert strides (elements)
 };
 
@@ -99,12 +100,25 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.moe_bs = a->moe_block_size;
   p.top_k = moe ? a->top_k : 1;
   p.mul_topk = moe && (a->flags & W4A16_F_MUL_TOPK_WEIGHTS);
+  p.n_sorted = moe ? (int)a->n_sorted : 0;
   p.b_estride = (a->size_k / 16) * (2 * a->size_n);
   p.s_estride = a->num_groups * a->size_n;
   p.z_estride = a->num_groups * (a->size_n / 8);
   p.k_estride = a->size_k;
   p.n_estride = a->size_n;
   return p;
+}
+
+// In-place MFMA on an accumulator pinned to AGPRs.  With 128 or 256 accumulators per lane the register allocator
+// otherwise assigns different registers to an MFMA's source and destination accumulator and fills the loop
+// with v_accvgpr moves (more of them than dequantisation instructions).  Source C == destination is the form
+// the matrix pipe forwards without extra wait states; results are only read again after the main loop.
+template <int DT>
+__device__ __forceinline__ void mfma_inplace(f32x4& acc, const u32x4& a, const u32x4& b) {
+  if constexpr (DT == DT_F16)
+    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  else
+    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 constexpr int RED_RS = 148;  // row stride (floats) of the 128-column reduction slab (4 mod 16: conflict-free)

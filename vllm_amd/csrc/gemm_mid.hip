@@ -1,0 +1,316 @@
+// W4A16 GEMM for gfx950 with 64-row tiles: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias), dense (64 < M, too few
+// rows or tiles for the 128-row prefill kernel) and MoE blocks of 64 sorted token slots
+// (the counterpart of the reference's thread_m_blocks = 4 configurations, csrc/moe/marlin_moe_wna16/ops.cu:451-512).
+//
+//   workgroup tile 64 rows x 512 columns, 4 wavefronts, each owning 64 rows x 128 columns (one column pair):
+//   4 m-blocks x 8 MFMA column groups = 32 v_mfma_f32_16x16x32 per k-step, 128 fp32 accumulators per lane in
+//   AGPRs and fewer than 128 VGPRs, so two workgroups share a compute unit (two wavefronts per SIMD): one
+//   wavefront's dequantisation and waits run under the other's MFMAs.
+//   weights      each wavefront streams its column pair global -> registers (128-bit loads, four k-steps in
+//                flight) and dequantises each Marlin word right before its 8 MFMAs, one operand register per MFMA
+//                (scale applied per element: the B operand equals the reference's half(q - z) * half(s)).
+//   activations  the workgroup stages 64 rows x 64 K (two k-steps) into LDS, double buffered, in MFMA fragment
+//                order (one conflict-free ds_read_b128 per operand); MoE rows are gathered through sorted_token_ids
+//                while staging.  One barrier per two k-steps.
+// Requirements (host-checked): K % 128 == 0, scales grouped or channelwise (no per-row g_idx), A's columns already
+// in weight order (dense act-order is gathered beforehand), MoE block size 64.
+#include <type_traits>
+
+#include "gemm_kernels.h"
+
+namespace w4a16 {
+
+constexpr int MD_MB = 4;     // m-blocks per tile
+constexpr int MD_BM = 64;    // rows per tile
+constexpr int MD_D = 4;      // weight k-steps in flight per wavefront
+constexpr int MD_ABUF = 2 * MD_MB * 64 * 16;            // one A buffer: 2 k-steps x 4 m-blocks x 64 lanes x 16 B
+constexpr int MD_SLABS = 4 * 16 * RED_RS * 4;           // four wavefront slabs of the epilogue
+constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_BM * 4;  // + C row of each tile row
+
+template <int DT, bool ZP, bool CHANNEL, bool MOE>
+__global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
+  constexpr bool UNIT = CHANNEL;
+  extern __shared__ __align__(16) unsigned char smem[];
+  int* s_crow = (int*)(smem + MD_SMEM - MD_BM * 4);
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
+
+  // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
+  // (MoE: neighbouring blocks mostly belong to the same expert)
+  const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
+  const int mt = blockIdx.x % mtiles, nt4 = blockIdx.x / mtiles;
+  const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
+  const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
+  const int row0 = mt * MD_BM;
+
+  const uint32_t* Bq = p.B;
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint32_t* Zp = p.Z;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  if (MOE) {
+    if (row0 >= *p.ntpp) return;
+    const int e = p.expert_ids[mt];
+    if (e < 0) return;  // expert of another rank
+    Bq += e * p.b_estride;
+    Sc += e * p.s_estride;
+    if (ZP) Zp += e * p.z_estride;
+    if (bias) bias += e * p.n_estride;
+  }
+  // which A row feeds tile row r and which C row receives it (-1: none)
+  auto tile_row_ids = [&](int r, int& src, int& dst) {
+    src = dst = -1;
+    if (MOE) {
+      const int id = p.sorted_ids[row0 + r];
+      if ((unsigned)id < (unsigned)p.c_rows) {
+        src = id / p.top_k;
+        dst = id;
+      }
+    } else if (row0 + r < p.M) {
+      src = dst = row0 + r;
+    }
+  };
+  if (t < MD_BM) {
+    int src, dst;
+    tile_row_ids(t, src, dst);
+    s_crow[t] = dst;
+  }
+
+  // ---- weights of this wavefront
+  const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
+  const int64_t b_row = p.N >> 1;
+  const u32x4* bp = (const u32x4*)Bq + nt * 32 + (4 * c + g);
+  const int64_t s_row = p.N >> 3;
+  const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
+  const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
+
+  // ---- activation staging: thread t loads piece (t & 7) of tile rows (t >> 3) + 32 i, i = 0..1
+  // (rows without a source read row 0 of A; their results are never stored)
+  const int piece = t & 7;
+  const uint16_t* arow[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    int src, dst;
+    tile_row_ids((t >> 3) + 32 * i, src, dst);
+    arow[i] = (const uint16_t*)p.A + (int64_t)(src < 0 ? 0 : src) * p.lda + piece * 8;
+  }
+  // LDS A layout: [buffer][k-step 2][m-block 4][lane 64][4 dwords]; the 16 bytes of (row, piece) are the K
+  // pairs 8*pp + 2q (pp = piece & 3), which belong to lane (q*16 + row%16), dword pp, of k-step piece >> 2.
+  uint32_t* lds = (uint32_t*)smem;
+  int a_wr[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = (t >> 3) + 32 * i;
+    a_wr[i] = (((piece >> 2) * MD_MB + (r >> 4)) * 64 + (r & 15)) * 4 + (piece & 3);
+  }
+  u32x4 areg[2];
+  // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
+  //  keeps the main loop free of branches)
+  auto load_a = [&](int chunk) {
+    chunk = min(chunk, p.total_ksteps / 2 - 1);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
+  };
+  auto store_a = [&](int buf) {
+    uint32_t* dst = lds + buf * (MD_ABUF / 4);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dst[a_wr[i] + q * 64] = areg[i][q];
+    }
+  };
+
+  struct Stage {
+    u32x4 b0, b1, sc;
+    uint32_t zq;
+  };
+  Stage st[MD_D];
+  auto issue = [&](Stage& s, int ks) {
+    ks = min(ks, p.total_ksteps - 1);
+    int gi = 0;
+    if (!CHANNEL) gi = ks / p.group_ksteps;
+    if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
+    if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    s.b0 = bp[(int64_t)(2 * ks) * b_row];
+    s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+  };
+  auto col_const = [&](const Stage& s, int w) {
+    uint32_t z0 = 8, z1 = 8;
+    if (ZP) {
+      z0 = (s.zq >> (4 * w)) & 0xf;
+      z1 = (s.zq >> (4 * w + 16)) & 0xf;
+    }
+    return make_col_const<DT, UNIT>(CHANNEL ? 0u : s.sc[w], z0, z1);
+  };
+
+  f32x4 acc[MD_MB][4][2];
+#pragma unroll
+  for (int mb = 0; mb < MD_MB; ++mb)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      acc[mb][w][0] = f32x4{0, 0, 0, 0};
+      acc[mb][w][1] = f32x4{0, 0, 0, 0};
+    }
+
+  const int nchunks = p.total_ksteps / 2;  // total_ksteps is a multiple of 4 (K % 128 == 0)
+
+  // ---- prologue
+  load_a(0);
+#pragma unroll
+  for (int j = 0; j < MD_D; ++j) issue(st[j], j);
+  store_a(0);
+  // B operands of two Marlin words: the one whose MFMAs are being issued and the one being dequantised
+  u32x4 ob[2][2];
+  {
+    const ColConst<DT> cc = col_const(st[0], 0);
+    dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], cc, ob[0][0], ob[0][1]);
+  }
+  __syncthreads();
+
+  // One k-step: per Marlin word w, 8 MFMAs on ob[w & 1]; after each MFMA one register of the following word's
+  // operands (word w + 1 of this k-step, or word 0 of the next k-step `nxt`) is dequantised into ob[(w + 1) & 1].
+  // The scheduling barriers keep the compiler from regrouping this into MFMA-only and VALU-only blocks.
+  auto kstep = [&](int buf, int kk, const Stage& cur, const Stage& nxt) {
+    const u32x4* abase = (const u32x4*)(lds + buf * (MD_ABUF / 4)) + (kk * MD_MB) * 64 + lane;
+    u32x4 af[MD_MB];
+#pragma unroll
+    for (int mb = 0; mb < MD_MB; ++mb) af[mb] = abase[mb * 64];
+    auto word = [&](auto w_tag) {
+      constexpr int w = decltype(w_tag)::value;
+      constexpr int wn = (w + 1) & 3;
+      const Stage& src = w == 3 ? nxt : cur;
+      const ColConst<DT> cc = col_const(src, wn);
+      const uint32_t xa = src.b0[wn], xb = src.b1[wn];
+      auto step = [&](auto j_tag) {
+        constexpr int J = decltype(j_tag)::value;
+        mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
+        const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        if constexpr (J < 4)
+          ob[wn & 1][0][J] = r;
+        else
+          ob[wn & 1][1][J - 4] = r;
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      step(std::integral_constant<int, 0>{});
+      step(std::integral_constant<int, 1>{});
+      step(std::integral_constant<int, 2>{});
+      step(std::integral_constant<int, 3>{});
+      step(std::integral_constant<int, 4>{});
+      step(std::integral_constant<int, 5>{});
+      step(std::integral_constant<int, 6>{});
+      step(std::integral_constant<int, 7>{});
+    };
+    word(std::integral_constant<int, 0>{});
+    word(std::integral_constant<int, 1>{});
+    word(std::integral_constant<int, 2>{});
+    word(std::integral_constant<int, 3>{});
+  };
+
+  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration
+#pragma unroll 1
+  for (int c0 = 0; c0 < nchunks; c0 += 2) {
+    const int ks0 = 2 * c0;
+    // chunk c0 in buffer 0
+    load_a(c0 + 1);
+    kstep(0, 0, st[0], st[1]);
+    issue(st[0], ks0 + 4);
+    kstep(0, 1, st[1], st[2]);
+    issue(st[1], ks0 + 5);
+    store_a(1);
+    __syncthreads();
+    // chunk c0+1 in buffer 1
+    load_a(c0 + 2);
+    kstep(1, 0, st[2], st[3]);
+    issue(st[2], ks0 + 6);
+    kstep(1, 1, st[3], st[0]);
+    issue(st[3], ks0 + 7);
+    store_a(0);
+    __syncthreads();
+  }
+
+  // ------------------------------------------------------------------------------ epilogue
+  // (the inline-asm MFMAs are opaque to the compiler's hazard logic: let the matrix pipe drain before the
+  //  accumulators are read)
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // per wavefront and m-block: accumulators -> private LDS slab [16 rows][RED_RS] -> 8-byte row stores.
+  // (the last barrier of the loop separates the slabs from the A buffers they overlay)
+  float* slab = (float*)smem + wv * (16 * RED_RS);
+  const int fc4 = (lane & 31) * 4;
+  const int fpos = fc4 + (fc4 >= 64 ? 8 : 0);
+  const int ncol = cp * 128 + fc4;
+  const bool fcol_ok = wave_on && ncol < p.N;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if (fcol_ok) {
+    const int base = ncol & ~31, cl = ncol & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  }
+#pragma unroll
+  for (int mb = 0; mb < MD_MB; ++mb) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) slab[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r16 = (lane >> 5) + 2 * i;
+      const int crow = s_crow[mb * 16 + r16];
+      f32x4 v = *(const f32x4*)(slab + r16 * RED_RS + fpos);
+      if (fcol_ok && crow >= 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+        if (MOE && p.mul_topk) {
+          const float tw = p.topk_w[crow];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] *= tw;
+        }
+        u32x2 o;
+        if constexpr (DT == DT_F16)
+          o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+        else
+          o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+        *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+typedef void (*mid_fn)(const KParams);
+
+template <int DT, bool MOE>
+static mid_fn pick_mid2(bool zp, bool channel) {
+  if (zp) return channel ? mid_kernel<DT, true, true, MOE> : mid_kernel<DT, true, false, MOE>;
+  return channel ? mid_kernel<DT, false, true, MOE> : mid_kernel<DT, false, false, MOE>;
+}
+
+int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
+  const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
+  const bool moe = (a->flags & W4A16_F_MOE) != 0;
+  mid_fn fn;
+  if (a->dtype == DT_F16)
+    fn = moe ? pick_mid2<DT_F16, true>(zp, channel) : pick_mid2<DT_F16, false>(zp, channel);
+  else
+    fn = moe ? pick_mid2<DT_BF16, true>(zp, channel) : pick_mid2<DT_BF16, false>(zp, channel);
+  KParams p = make_kparams(a, pl);
+  const int64_t grid = (int64_t)pl.tiles;
+  if (grid <= 0) return 0;
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), MD_SMEM, stream, p);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace w4a16

@@ -12,7 +12,7 @@ struct Plan {
   int mtiles, ncp, tiles;
   int total_ksteps, splits, kps;  // k-steps of 32 rows; K splits; k-steps per split
   int xcd_map;
-  int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel
+  int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel, 3: 64-row ("mid") kernel
   int tn;    // tile width in columns (128; the decode kernel also has 64)
   int64_t ctmp_bytes;  // fp32 split-K partials
   int64_t atmp_bytes;  // column-permuted copy of A (act-order in front of the prefill kernel), after the partials
@@ -21,5 +21,6 @@ struct Plan {
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
+int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 
 }  // namespace w4a16
