@@ -177,6 +177,26 @@ def _unpack_rows_gpu(p):  # GPTQ int32 [K/8, N] -> [K, N]
     return (((p.to(torch.int64) & 0xFFFFFFFF).unsqueeze(1) >> sh) & 0xF).reshape(-1, p.shape[1]).to(torch.int32)
 
 
+def bench_repack(ops, dev):
+    """Load-time repack of the four layers (GPTQ and AWQ checkpoint layouts -> Marlin layout): K*N/2 bytes read and
+    K*N/2 written per call, against the HBM peak."""
+    out = {}
+    empty = torch.empty(0, dtype=torch.int32, device=dev)
+    for name, (k, n) in LAYERS.items():
+        g = torch.Generator(device=dev).manual_seed(9)
+        gq = torch.randint(-2**31, 2**31 - 1, (k // 8, n), generator=g, device=dev, dtype=torch.int32)
+        aq = torch.randint(-2**31, 2**31 - 1, (k, n // 8), generator=g, device=dev, dtype=torch.int32)
+        for kind, fn in (("gptq", lambda: ops.gptq_marlin_repack(gq, empty, k, n, 4)),
+                         ("awq", lambda: ops.awq_marlin_repack(aq, k, n, 4))):
+            sec = time_graph([fn] * 8, reps=3, warmup=1) / 8
+            by = k * n  # bytes moved: half read, half written
+            out[f"{kind}_{name}"] = {"k": k, "n": n, "us": sec * 1e6, "GBps": by / sec / 1e9,
+                                     "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS}
+            print(f"[detail] {kind} repack {name}: {sec * 1e6:.1f} us, {by / sec / 1e9:.0f} GB/s = "
+                  f"{100 * by / sec / 1e9 / HBM_PEAK_GBPS:.1f}% HBM", file=sys.stderr, flush=True)
+    return out
+
+
 def bench_act_order(ops, wtype, dev, workspace):
     """BASELINE config 4: down_proj (K=14336, N=4096), g128, desc_act, fp16, M in {1, 16, 512}."""
     k, n = LAYERS["down"]
@@ -409,6 +429,7 @@ def main():
         torch.cuda.empty_cache()
         detail["mixtral_moe_fp16_gptq"] = bench_moe(ops, scalar_types.uint4b8, dev)
         torch.cuda.empty_cache()
+        detail["repack"] = bench_repack(ops, dev)
         result["detail"] = detail
         if args.table:
             with open(args.table, "w") as f:

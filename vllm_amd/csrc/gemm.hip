@@ -82,6 +82,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
   pl.total_ksteps = (int)(a->size_k / 32);
   const int cus = num_cus();
+  // Overrides for tuning experiments (unset in production): force the number of K splits, the decode tile width,
+  // or the kernel kind (0 skinny, 1 decode, 2 prefill, 3 64-row); W4A16_DEBUG=1 prints the chosen plan.
   static const int forced_splits = env_int("W4A16_SPLITS", 0);
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
@@ -92,9 +94,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   pl.atmp_bytes = (act_order && !moe) ? a->size_m * a->size_k * 2 : 0;
   const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
-  static const int fat_min_m = env_int("W4A16_FAT_MIN_M", 128);
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
-  if (!moe && a->size_m >= fat_min_m && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  if (!moe && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
@@ -141,9 +142,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
                             (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
 
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these
-  // kernels.  One 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~21 GB/s on a 64-column
+  // kernels.  One 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~20 GB/s on a 64-column
   // strip with 16-row tiles (instruction-issue bound), ~12 / ~9 GB/s with 32- / 64-row tiles (dequantisation
-  // per element); the whole chip ~4.7 TB/s; summing K-splits across workgroups adds ~3 us of dependent
+  // per element); the whole chip ~4.7 TB/s; summing K-splits across workgroups adds ~2.2 us of dependent
   // device-scope round trips plus the last workgroup's pass over the partial tiles.  Only one such workgroup
   // fits a compute unit, so a grid larger than the number of compute units runs in rounds.  Each split needs
   // >= 1 stage per wavefront and one workspace counter per tile.
@@ -165,7 +166,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       const int64_t tiles = mtiles * ncol_tiles;
       if (tiles <= 0 || tiles >= (1LL << 31) / 64) continue;
       const double bytes = (double)tiles * a->size_k * tn / 2.0;
-      const double wg_rate = mb == 1 ? (tn == 64 ? 21e3 : 33e3) : mb == 2 ? 12e3 : 9e3;  // bytes per us
+      const double wg_rate = mb == 1 ? (tn == 64 ? 20e3 : 33e3) : mb == 2 ? 12e3 : 9e3;  // bytes per us
       const double chip_rate = 4.7e6;
       const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
       const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
@@ -179,7 +180,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
         double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
         if (rate > chip_rate) rate = chip_rate;
         // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
-        const double t_fix = sp > 1 ? 2.8 + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
+        const double t_fix = sp > 1 ? 2.2 + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
         const double t = bytes / rate + t_fix;
         if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, mb, t};
       }

@@ -23,7 +23,6 @@ struct KParams {
   int ncp;           // column pairs = ceil(N / 128)
   int splits, ksteps_per_split, total_ksteps;
   int xcd_map;
-  int fix_mode;  // debugging switches (0 in production)
   int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
   // MoE
   const int32_t* sorted_ids;
@@ -46,7 +45,7 @@ __device__ __forceinline__ void store_coherent2(float* ptr, float f0, float f1) 
   const u64 a = (u64)__builtin_bit_cast(uint32_t, f0) | ((u64)__builtin_bit_cast(uint32_t, f1) << 32);
   __hip_atomic_store((u64*)ptr, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void store_coherent(float* ptr, f32x4 v, int /*mode*/ = 0) {
+__device__ __forceinline__ void store_coherent(float* ptr, f32x4 v) {
   // (elements are copied to scalars first: bit-casting a vector element directly reads element 0)
   const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
   store_coherent2(ptr, f0, f1);
@@ -58,7 +57,7 @@ __device__ __forceinline__ void load_coherent2(const float* ptr, float& f0, floa
   f0 = __builtin_bit_cast(float, (uint32_t)a);
   f1 = __builtin_bit_cast(float, (uint32_t)(a >> 32));
 }
-__device__ __forceinline__ f32x4 load_coherent(const float* ptr, int /*mode*/ = 0) {
+__device__ __forceinline__ f32x4 load_coherent(const float* ptr) {
   float f0, f1, f2, f3;
   load_coherent2(ptr, f0, f1);
   load_coherent2(ptr + 2, f2, f3);
@@ -90,7 +89,6 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.ksteps_per_split = pl.kps;
   p.total_ksteps = pl.total_ksteps;
   p.xcd_map = pl.xcd_map;
-  p.fix_mode = 0;
   p.tn = pl.tn;
   p.sorted_ids = a->sorted_token_ids;
   p.expert_ids = a->expert_ids;

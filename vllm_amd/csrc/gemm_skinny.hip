@@ -22,6 +22,8 @@
 // once per column pair (from L2), split partials move 2 * splits * M * N * 4 bytes.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "gemm_kernels.h"
 
 namespace w4a16 {
@@ -504,9 +506,11 @@ int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
   KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);
   if (smem > 64 * 1024) {
-    // more than 64 KiB of dynamic LDS has to be allowed per kernel function; do it once per function
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel function; once per function and process
+    static std::mutex mu;
     static const void* allowed[64];
     static int n_allowed = 0;
+    std::lock_guard<std::mutex> lock(mu);
     bool seen = false;
     for (int i = 0; i < n_allowed; ++i) seen |= allowed[i] == (const void*)fn;
     if (!seen) {
