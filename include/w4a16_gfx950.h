@@ -32,7 +32,7 @@ enum {
  * vllm/scalar_type.py:136-164, csrc/core/scalar_type.hpp:143-160) */
 enum { W4A16_WTYPE_U4B8 = 0, W4A16_WTYPE_U4 = 1 };
 /* activation / output / scale element type */
-enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1 };
+enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1, W4A16_DTYPE_F32 = 2 /* router logits only */ };
 
 int w4a16_abi_version(void);
 const char* w4a16_last_error(void);
@@ -126,6 +126,14 @@ int w4a16_moe_sum(const void* in, void* out, int64_t tokens, int32_t top_k, int6
  * csrc/torch_bindings.cpp:118): out[t, j] = silu(in[t, j]) * in[t, d + j]. */
 int w4a16_silu_and_mul(const void* in, void* out, int64_t tokens, int64_t d, int32_t dtype,
                        void* stream);
+
+/* Replaces torch.ops._moe_C.topk_softmax (csrc/moe/topk_softmax_kernels.cu:676-705, schema
+ * csrc/moe/torch_bindings.cpp:6-8): fp32 softmax over num_experts router logits per token (fp16 / bf16 / fp32),
+ * top-k by repeated arg-max (ties: lowest index), weights optionally renormalised to sum to 1;
+ * token_expert_indices[t, k] = k * num_tokens + t.  All outputs [num_tokens, topk]. */
+int w4a16_topk_softmax(const void* gating_output, int32_t gating_dtype, float* topk_weights,
+                       int32_t* topk_ids, int32_t* token_expert_indices, int64_t num_tokens,
+                       int32_t num_experts, int32_t topk, int32_t renormalize, void* stream);
 
 #ifdef __cplusplus
 }

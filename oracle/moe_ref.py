@@ -9,7 +9,8 @@ Pinned by (tests/test_oracle_moe.py): the docstring example (topk_ids
 [[2,3,4],[1,2,4],[1,3,4],[1,2,3]], block 4 -> sorted ids
 [3,6,9,12,0,4,10,12,1,7,11,12,2,5,8,12] once the unused expert 0 is skipped), the
 invariants of test_moe_align_block_size.py:210-231, a brute-force per-token loop for the
-experts computation, and moe_gemm_ref == dense gemm_ref per expert on gathered rows.
+experts computation, moe_gemm_ref == dense gemm_ref per expert on gathered rows, and for topk_softmax a
+hand-computed three-expert case with a tie plus agreement with torch.topk on tie-free inputs.
 """
 import torch
 
@@ -40,6 +41,30 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     if expert_map is not None:
         expert_ids = expert_map[expert_ids.long()].to(torch.int32)
     return sorted_ids, expert_ids, total
+
+
+def topk_softmax(gating_output: torch.Tensor, topk: int, renormalize: bool):
+    """Routing as the reference's topk_softmax op (csrc/moe/topk_softmax_kernels.cu:127-211): fp32 softmax,
+    k rounds of arg-max with ties going to the lowest expert index, optional renormalisation (zero sum -> divide
+    by 1), token_expert_indices[t, k] = k * num_tokens + t.  Scalar loops: small cases only."""
+    t, e = gating_output.shape
+    p = torch.softmax(gating_output.float(), dim=-1)
+    w = torch.zeros(t, topk, dtype=torch.float32)
+    ids = torch.zeros(t, topk, dtype=torch.int32)
+    src = torch.zeros(t, topk, dtype=torch.int32)
+    for r in range(t):
+        taken = set()
+        for k in range(topk):
+            best, be = -1.0, -1
+            for x in range(e):
+                if x not in taken and float(p[r, x]) > best:
+                    best, be = float(p[r, x]), x
+            taken.add(be)
+            w[r, k], ids[r, k], src[r, k] = p[r, be], be, k * t + r
+        if renormalize:
+            d = w[r].sum()
+            w[r] = w[r] / (d if d > 0 else 1.0)
+    return w, ids, src
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:

@@ -74,6 +74,41 @@ def test_silu_and_mul(dev, dtype, m, d):
     assert torch.allclose(got, mr.silu_and_mul(x.float()), rtol=4 * eps, atol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,e,topk", [(1, 8, 2), (33, 8, 2), (7, 60, 6), (128, 64, 8), (5, 256, 8), (3, 1000, 4)])
+@pytest.mark.parametrize("renorm", [False, True])
+def test_topk_softmax(dev, dtype, t, e, topk, renorm):
+    from vllm_amd.fused_moe import fused_topk
+    g = torch.Generator().manual_seed(t + e)
+    logits = (torch.randn(t, e, generator=g) * 2).to(dtype)
+    w, ids, src = fused_topk(torch.empty(t, 4, device=dev), logits.to(dev), topk, renorm)
+    p = torch.softmax(logits.float(), dim=-1)
+    tw, ti = torch.topk(p, topk)
+    if renorm:
+        tw = tw / tw.sum(-1, keepdim=True)
+    assert w.dtype == torch.float32 and ids.dtype == torch.int32
+    # 16-bit logits can tie exactly: compare the selected probabilities, and the ids wherever they are unambiguous
+    torch.testing.assert_close(w.cpu(), tw, rtol=2e-5, atol=1e-7)
+    sel = torch.gather(p, 1, ids.cpu().long())
+    assert torch.equal(sel, torch.gather(p, 1, ti))
+    for r in range(t):
+        assert len(set(ids[r].tolist())) == topk
+    assert src.cpu().tolist() == [[k * t + r for k in range(topk)] for r in range(t)]
+    if t * e <= 2048:
+        ow, oi, _ = mr.topk_softmax(logits, topk, renorm)     # scalar oracle incl. lowest-index tie-break
+        assert torch.equal(ids.cpu(), oi)
+        torch.testing.assert_close(w.cpu(), ow, rtol=2e-5, atol=1e-7)
+
+
+def test_topk_softmax_ties_take_lowest_index(dev):
+    from vllm_amd.fused_moe import fused_topk
+    logits = torch.zeros(2, 130, device=dev)
+    logits[1, 70] = 1.0
+    w, ids, _ = fused_topk(torch.empty(2, 4, device=dev), logits, 3, True)
+    assert ids.cpu().tolist() == [[0, 1, 2], [70, 0, 1]]
+    assert torch.allclose(w[0].cpu(), torch.full((3,), 1 / 3))
+
+
 # ------------------------------------------------------------------------------------- MoE GEMM
 def make_experts(e, k, n, group, dtype, has_zp, act_order, seed):
     layers = [make_layer(k, n, group, dtype, has_zp=has_zp, act_order=act_order, seed=seed + i, w_std=0.1) for i in range(e)]

@@ -94,3 +94,19 @@ def test_moe_gemm_ref_is_dense_gemm_per_expert():
                 if mul:
                     want = want * tw[t, s]
                 assert torch.allclose(out[t * topk + s], want, atol=1e-5)
+
+
+def test_topk_softmax_hand_case_and_torch_agreement():
+    import math
+    # logits (0, ln 2, ln 2, -inf-ish): probabilities 0.2, 0.4, 0.4, ~0; the tie goes to the lower index
+    g = torch.tensor([[0.0, math.log(2.0), math.log(2.0), -50.0]])
+    w, ids, src = mr.topk_softmax(g, 2, False)
+    assert ids.tolist() == [[1, 2]] and src.tolist() == [[0, 1]]
+    assert torch.allclose(w, torch.tensor([[0.4, 0.4]]), atol=1e-6)
+    w, ids, _ = mr.topk_softmax(g, 3, True)
+    assert ids.tolist() == [[1, 2, 0]] and torch.allclose(w, torch.tensor([[0.4, 0.4, 0.2]]), atol=1e-6)
+    x = torch.randn(9, 16, generator=torch.Generator().manual_seed(3))
+    w, ids, src = mr.topk_softmax(x, 4, True)
+    tw, ti = torch.topk(torch.softmax(x, -1), 4)
+    assert torch.equal(ids.long(), ti) and torch.allclose(w, tw / tw.sum(-1, keepdim=True), atol=1e-6)
+    assert src.tolist() == [[k * 9 + r for k in range(4)] for r in range(9)]

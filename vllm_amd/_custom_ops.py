@@ -4,7 +4,8 @@ Defines (when nothing else has) and implements, for the CUDA dispatch key (= HIP
 PyTorch-ROCm), the operators the reference reaches through `vllm/_custom_ops.py`:
 
   _C::gptq_marlin_repack, _C::awq_marlin_repack, _C::gptq_marlin_gemm, _C::permute_cols,
-  _C::silu_and_mul, _moe_C::moe_wna16_marlin_gemm, _moe_C::moe_align_block_size, _moe_C::moe_sum
+  _C::silu_and_mul, _moe_C::moe_wna16_marlin_gemm, _moe_C::moe_align_block_size, _moe_C::moe_sum,
+  _moe_C::topk_softmax
 
 with the reference's schemas (csrc/torch_bindings.cpp:118, 312-336; csrc/moe/torch_bindings.cpp:13-23, 63-75),
 plus fake (meta) implementations for tracing (reference vllm/_custom_ops.py:553-576, 1179-1218,
@@ -49,6 +50,8 @@ _MOE_SCHEMAS = {
     "moe_align_block_size": "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, "
                             "Tensor! sorted_token_ids, Tensor! experts_ids, Tensor! num_tokens_post_pad) -> ()",
     "moe_sum": "moe_sum(Tensor input, Tensor! output) -> ()",
+    "topk_softmax": "topk_softmax(Tensor! topk_weights, Tensor! topk_indices, Tensor! token_expert_indices, "
+                    "Tensor gating_output, bool renormalize) -> ()",
 }
 
 
@@ -357,6 +360,28 @@ def _silu_and_mul_impl(result, input):
                                                    _dtype_code(input.dtype), _stream(input.device)))
 
 
+def _topk_softmax_impl(topk_weights, topk_indices, token_expert_indices, gating_output, renormalize):
+    _check(gating_output.is_cuda and gating_output.is_contiguous() and gating_output.dim() == 2,
+           "gating_output must be a contiguous [num_tokens, num_experts] GPU tensor")
+    num_tokens, num_experts = gating_output.shape
+    topk = topk_weights.size(-1)
+    _check(topk_weights.dtype == torch.float32 and topk_weights.is_contiguous() and
+           tuple(topk_weights.shape) == (num_tokens, topk), "topk_weights must be fp32 [num_tokens, topk]")
+    _check(token_expert_indices.dtype == torch.int32 and token_expert_indices.is_contiguous() and
+           tuple(token_expert_indices.shape) == (num_tokens, topk), "token_expert_indices must be int32 [num_tokens, topk]")
+    _check(tuple(topk_indices.shape) == (num_tokens, topk) and topk_indices.is_contiguous(), "topk_indices shape mismatch")
+    code = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32}.get(
+        gating_output.dtype)
+    _check(code is not None, "gating_output must be fp16, bf16 or fp32")
+    ids = topk_indices if topk_indices.dtype == torch.int32 else torch.empty_like(topk_indices, dtype=torch.int32)
+    with torch.cuda.device(gating_output.device):
+        _lib.check(_lib.load().w4a16_topk_softmax(
+            _ptr(gating_output), code, _ptr(topk_weights), _ptr(ids), _ptr(token_expert_indices), num_tokens,
+            num_experts, topk, int(bool(renormalize)), _stream(gating_output.device)))
+    if ids is not topk_indices:
+        topk_indices.copy_(ids)
+
+
 # ------------------------------------------------------------------------------------- fakes
 def _gemm_fake(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none,
                g_idx_or_none, perm_or_none, workspace, b_q_type, size_m, size_n, size_k,
@@ -391,6 +416,7 @@ _IMPLS = {
         "moe_wna16_marlin_gemm": (_moe_wna16_marlin_gemm_impl, _moe_gemm_fake),
         "moe_align_block_size": (_moe_align_block_size_impl, lambda *a: None),
         "moe_sum": (_moe_sum_impl, lambda input, output: None),
+        "topk_softmax": (_topk_softmax_impl, lambda *a: None),
     },
 }
 _SCHEMAS = {"_C": _C_SCHEMAS, "_moe_C": _MOE_SCHEMAS}
@@ -493,3 +519,8 @@ def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, ex
 
 def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
     torch.ops._moe_C.moe_sum(input, output)
+
+
+def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, token_expert_indices: torch.Tensor,
+                 gating_output: torch.Tensor, renormalize: bool = False) -> None:
+    torch.ops._moe_C.topk_softmax(topk_weights, topk_ids, token_expert_indices, gating_output, renormalize)

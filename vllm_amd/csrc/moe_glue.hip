@@ -135,6 +135,94 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
   }
 }
 
+
+// Routing: fp32 softmax over the experts of one token, then top-k by repeated arg-max (ties -> lowest expert
+// index), as the reference's topk_softmax (csrc/moe/topk_softmax_kernels.cu:127-211, 676-705):
+// weights are the softmax probabilities of the chosen experts, optionally renormalised to sum to 1
+// (a zero sum divides by 1); token_expert_indices[t, k] = k * num_tokens + t.
+// One wavefront per token; lane l holds experts l, l + 64, ... (at most TOPK_PER_LANE of them) in registers.
+constexpr int TOPK_PER_LANE = 16;  // up to 1024 experts
+
+template <typename T>
+__device__ __forceinline__ float gate_to_f32(T v);
+template <>
+__device__ __forceinline__ float gate_to_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float gate_to_f32<_Float16>(_Float16 v) { return (float)v; }
+template <>
+__device__ __forceinline__ float gate_to_f32<__bf16>(__bf16 v) { return (float)v; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ gating, float* __restrict__ weights,
+                                                           int32_t* __restrict__ ids, int32_t* __restrict__ src_rows,
+                                                           int num_tokens, int num_experts, int topk, int renormalize) {
+  const int lane = threadIdx.x & 63;
+  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tok >= num_tokens) return;
+  const T* row = gating + (int64_t)tok * num_experts;
+  float v[TOPK_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < TOPK_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < num_experts ? gate_to_f32<T>(row[e]) : -INFINITY;
+    mx = fmaxf(mx, v[i]);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < TOPK_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < num_experts ? expf(v[i] - mx) : 0.f;
+    sum += v[i];
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+#pragma unroll
+  for (int i = 0; i < TOPK_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < num_experts ? v[i] / sum : -1.f;  // probabilities are >= 0: -1 marks "not a candidate"
+  }
+  float selected = 0.f;
+  for (int k = 0; k < topk; ++k) {
+    float bv = -1.f;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) {  // ascending expert index inside the lane: strict > keeps the lowest
+      if (v[i] > bv) {
+        bv = v[i];
+        be = lane + 64 * i;
+      }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const float ov = __shfl_xor(bv, d, 64);
+      const int oe = __shfl_xor(be, d, 64);
+      if (ov > bv || (ov == bv && oe < be)) {
+        bv = ov;
+        be = oe;
+      }
+    }
+    if (lane == 0) {
+      weights[(int64_t)tok * topk + k] = bv;
+      ids[(int64_t)tok * topk + k] = be;
+      src_rows[(int64_t)tok * topk + k] = k * num_tokens + tok;
+    }
+    selected += bv;
+    if ((be & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < TOPK_PER_LANE; ++i)
+        if (i == (be >> 6)) v[i] = -1.f;
+    }
+  }
+  // (lane 0 wrote the weights, so lane 0 rescales them: same-thread program order)
+  if (renormalize && lane == 0) {
+    const float denom = selected > 0.f ? selected : 1.f;
+    for (int k = 0; k < topk; ++k) weights[(int64_t)tok * topk + k] /= denom;
+  }
+}
+
 }  // namespace w4a16
 
 using namespace w4a16;
@@ -187,6 +275,32 @@ extern "C" int w4a16_silu_and_mul(const void* in, void* out, int64_t tokens, int
     silu_and_mul_kernel<DT_F16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, d / 8);
   else
     silu_and_mul_kernel<DT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, total8, d / 8);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_topk_softmax(const void* gating_output, int32_t gating_dtype, float* topk_weights,
+                                  int32_t* topk_ids, int32_t* token_expert_indices, int64_t num_tokens,
+                                  int32_t num_experts, int32_t topk, int32_t renormalize, void* stream) {
+  W4A16_CHECK(gating_output && topk_weights && topk_ids && token_expert_indices, "null pointer");
+  W4A16_CHECK(num_experts >= 1 && num_experts <= 64 * TOPK_PER_LANE, "num_experts = %d must be in [1, %d]", num_experts,
+              64 * TOPK_PER_LANE);
+  W4A16_CHECK(topk >= 1 && topk <= num_experts, "topk = %d must be in [1, num_experts]", topk);
+  W4A16_CHECK(num_tokens >= 0 && num_tokens < (1LL << 30), "bad num_tokens");
+  if (num_tokens == 0) return 0;
+  const unsigned grid = (unsigned)ceil_div(num_tokens, 4);
+  hipStream_t st = (hipStream_t)stream;
+  if (gating_dtype == W4A16_DTYPE_F16)
+    topk_softmax_kernel<_Float16><<<grid, 256, 0, st>>>((const _Float16*)gating_output, topk_weights, topk_ids,
+                                                       token_expert_indices, (int)num_tokens, num_experts, topk, renormalize);
+  else if (gating_dtype == W4A16_DTYPE_BF16)
+    topk_softmax_kernel<__bf16><<<grid, 256, 0, st>>>((const __bf16*)gating_output, topk_weights, topk_ids,
+                                                     token_expert_indices, (int)num_tokens, num_experts, topk, renormalize);
+  else if (gating_dtype == W4A16_DTYPE_F32)
+    topk_softmax_kernel<float><<<grid, 256, 0, st>>>((const float*)gating_output, topk_weights, topk_ids,
+                                                    token_expert_indices, (int)num_tokens, num_experts, topk, renormalize);
+  else
+    return fail(W4A16_EINVAL, "gating_output must be fp16, bf16 or fp32");
   W4A16_HIP(hipGetLastError());
   return 0;
 }
