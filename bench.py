@@ -29,9 +29,9 @@ LAYERS = {"qkv": (4096, 6144), "o": (4096, 4096), "gate_up": (4096, 28672), "dow
 GROUP = 128
 # HBM bytes per launch of the headline step's GEMM kernel (average of the four launches at M=16), from two
 # `rocprofv3 --pmc` runs of `bench.py --pmc-probe` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same
-# counter reads for the 256 MiB device copy in that run (FETCH_SIZE reads 0.5 KiB per KiB copied, WRITE_SIZE
-# 1.0): qkv 13912+192, o 10648+1162, gate_up 60436+896, down 34376+1162 KiB.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = (13912 + 192 + 10648 + 1162 + 60436 + 896 + 34376 + 1162) * 1024 / 4
+# counter reads for the 256 MiB device copy in that run (FETCH_SIZE reads 0.5 per KiB copied, WRITE_SIZE 1.0):
+# read + written KiB: qkv 14629 + 969, o 10648 + 1162, gate_up 60436 + 896, down 34377 + 1162.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = (14629 + 969 + 10648 + 1162 + 60436 + 896 + 34377 + 1162) * 1024 / 4
 
 
 def algorithmic_bytes(m, k, n, zp=False, act_order=False):
@@ -198,7 +198,7 @@ def bench_repack(ops, dev):
 
 
 def bench_act_order(ops, wtype, dev, workspace):
-    """BASELINE config 4: down_proj (K=14336, N=4096), g128, desc_act, fp16, M in {1, 16, 512}."""
+    """GPTQ act-order case: down_proj (K=14336, N=4096), g128, desc_act, fp16, M in {1, 16, 512}."""
     k, n = LAYERS["down"]
     base = make_gptq_actorder_layer(ops, k, n, torch.float16, dev, 21)
     ncopy = copies_needed(base["q"].numel() * 4)
@@ -224,7 +224,7 @@ def bench_act_order(ops, wtype, dev, workspace):
 
 
 def bench_moe(ops, wtype, dev):
-    """BASELINE config 5: Mixtral-8x7B fused MoE (8 experts, hidden 4096, intermediate 14336, top-2), uint4b8 g128
+    """Mixtral-8x7B fused MoE (8 experts, hidden 4096, intermediate 14336, top-2), uint4b8 g128
     fp16, T in {16, 512, 4096}; one call = align + GEMM1 + SiLU-and-mul + GEMM2 + top-k sum."""
     from vllm_amd.fused_marlin_moe import fused_marlin_moe
     e, hid, inter, topk = 8, 4096, 14336, 2
