@@ -30,7 +30,7 @@ enum {
 
 /* weight types (decoded from the reference's ScalarType ids by the host layer,
  * vllm/scalar_type.py:136-164, csrc/core/scalar_type.hpp:143-160) */
-enum { W4A16_WTYPE_U4B8 = 0, W4A16_WTYPE_U4 = 1 };
+enum { W4A16_WTYPE_U4B8 = 0, W4A16_WTYPE_U4 = 1, W4A16_WTYPE_U8B128 = 2 };
 /* activation / output / scale element type */
 enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1, W4A16_DTYPE_F32 = 2 /* router logits only */ };
 
@@ -39,15 +39,17 @@ const char* w4a16_last_error(void);
 
 /* Replaces torch.ops._C.gptq_marlin_repack
  * (csrc/quantization/gptq_marlin/gptq_marlin_repack.cu:251-322, schema csrc/torch_bindings.cpp:327-329).
- * b_q_weight: int32 [size_k/8, size_n] GPTQ packing (nibble i of word (r,n) = q[8r+i, n]).
+ * b_q_weight: int32 [size_k/8, size_n] GPTQ packing (nibble i of word (r,n) = q[8r+i, n]);
+ *             num_bits = 8: int32 [size_k/4, size_n], byte i of word (r,n) = q[4r+i, n].
  * perm: int32 [size_k] source-row order (act-order) or NULL.
- * out: int32 [size_k/16, 2*size_n] Marlin layout. */
+ * out: int32 [size_k/16, 2*size_n] Marlin layout (num_bits = 8: [size_k/16, 4*size_n]). */
 int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm, uint32_t* out,
                              int64_t size_k, int64_t size_n, int num_bits, void* stream);
 
 /* Replaces torch.ops._C.awq_marlin_repack
  * (csrc/quantization/gptq_marlin/awq_marlin_repack.cu:189-248, schema csrc/torch_bindings.cpp:333-335).
- * b_q_weight: int32 [size_k, size_n/8] AWQ packing (nibble t of word (k,c) = q[k, 8c+{0,2,4,6,1,3,5,7}[t]]). */
+ * b_q_weight: int32 [size_k, size_n/8] AWQ packing (nibble t of word (k,c) = q[k, 8c+{0,2,4,6,1,3,5,7}[t]]);
+ *             num_bits = 8: int32 [size_k, size_n/4], byte t of word (k,c) = q[k, 4c+{0,2,1,3}[t]]. */
 int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
                             int64_t size_n, int num_bits, void* stream);
 

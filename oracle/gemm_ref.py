@@ -19,7 +19,7 @@ dequant_checkpoint == w_ref likewise; fp32 matmul is torch's.
 import numpy as np
 import torch
 
-from .marlin_layout import (marlin_unpack_weights, marlin_unpack_zero_points,
+from .marlin_layout import (marlin_unpack_weights, marlin_unpack_weights8, marlin_unpack_zero_points,
                             marlin_unpermute_scales)
 from .quant_utils import awq_unpack, unpack_rows
 
@@ -35,13 +35,14 @@ def _expand_groups(t: torch.Tensor, size_k: int, g_idx=None) -> torch.Tensor:
     return t.repeat_interleave(size_k // g, dim=0)
 
 
-def dequant_marlin(b_q_weight, b_scales, b_zeros, g_idx, size_k, size_n, bias8: bool, dtype):
+def dequant_marlin(b_q_weight, b_scales, b_zeros, g_idx, size_k, size_n, bias8: bool, dtype, num_bits: int = 4):
     """Marlin operands -> dense w[K, N] (row i = Marlin row i, i.e. after act-order sort).
 
-    b_scales [G, N] Marlin-permuted; b_zeros int32 [G, N/8] Marlin-packed or None;
+    b_scales [G, N] Marlin-permuted; b_zeros int32 [G, N/8] Marlin-packed or None; bias8: the stored value
+    carries the type's bias (8 for uint4b8, 128 for uint8b128);
     g_idx: sorted group id per Marlin row (only when the scale row is looked up per row).
     """
-    q = marlin_unpack_weights(b_q_weight)
+    q = marlin_unpack_weights(b_q_weight) if num_bits == 4 else marlin_unpack_weights8(b_q_weight)
     assert tuple(q.shape) == (size_k, size_n)
     num_groups = b_scales.shape[0]
     grouped = num_groups > 1
@@ -52,7 +53,7 @@ def dequant_marlin(b_q_weight, b_scales, b_zeros, g_idx, size_k, size_n, bias8: 
         z_full = _expand_groups(z, size_k, g_idx)
         qz = q - z_full
     else:
-        qz = q - (8 if bias8 else 0)
+        qz = q - ((8 if num_bits == 4 else 128) if bias8 else 0)
     return qz.to(dtype) * s_full
 
 

@@ -9,6 +9,9 @@ Reference statements followed:
   bias      marlin_utils.py:301-305
   zeros     marlin_utils.py:326-370 (marlin_zero_points, awq_to_marlin_zero_points)
 
+The 8-bit weight layout (uint8b128) has the same two formulations (`marlin_weights_closed_form8`,
+`marlin_weights_perm_table(num_bits=8)`) and is pinned the same way (tests/test_oracle_layout.py).
+
 Two independent formulations of the weight layout are kept on purpose:
 `marlin_weights_closed_form` (index arithmetic per output nibble) and
 `marlin_weights_perm_table` (tile transpose + 1024-entry permutation + pack).
@@ -59,6 +62,51 @@ def marlin_weights_closed_form(q, perm=None) -> torch.Tensor:
     return _to_i32_tensor(out.reshape(k // 16, 2 * n))
 
 
+def marlin_weights_closed_form8(q, perm=None) -> torch.Tensor:
+    """8-bit layout by direct index arithmetic (gptq_marlin_repack.cu:119-203 with num_bits = 8).
+
+    Output int32 [K/16, 4N].  Per k-tile and 64-column n-tile 256 words; word nt*256 + th*8 + 2*w + half
+    (th in [0,32), w in [0,4), half in {0,1}) holds, with r = 2*(th % 4), c = th // 4, n = 64*nt + 16*w + c + 8*half,
+    k0 = 16*kt + r, the bytes q[k0 + (0, 8, 1, 9)[j], n] for j = 0..3."""
+    qa = _u32(q)
+    k, n = qa.shape
+    assert k % TILE_K == 0 and n % TILE_N == 0
+    if perm is not None and len(perm) > 0:
+        qa = qa[np.asarray(perm, dtype=np.int64)]
+    kt = np.arange(k // 16)[:, None, None, None, None]
+    nt = np.arange(n // 64)[None, :, None, None, None]
+    th = np.arange(32)[None, None, :, None, None]
+    w = np.arange(4)[None, None, None, :, None]
+    half = np.arange(2)[None, None, None, None, :]
+    k0 = 16 * kt + 2 * (th % 4)
+    nn = 64 * nt + 16 * w + th // 4 + 8 * half
+    out = np.zeros((k // 16, n // 64, 32, 4, 2), dtype=np.uint32)
+    for j, dk in enumerate((0, 8, 1, 9)):
+        kk, n2 = np.broadcast_arrays(k0 + dk, nn)
+        out |= (qa[kk, n2] & 0xFF) << np.uint32(8 * j)
+    return _to_i32_tensor(out.reshape(k // 16, 4 * n))
+
+
+def marlin_unpack_weights8(marlin_w) -> torch.Tensor:
+    """Inverse of the 8-bit layout: int32 [K/16, 4N] -> int32 [K, N] bytes."""
+    wa = _u32(marlin_w)
+    kt_n, words = wa.shape
+    n = words // 4
+    out = np.zeros((kt_n * 16, n), dtype=np.int32)
+    wa = wa.reshape(kt_n, n // 64, 32, 4, 2)
+    kt = np.arange(kt_n)[:, None, None, None, None]
+    nt = np.arange(n // 64)[None, :, None, None, None]
+    th = np.arange(32)[None, None, :, None, None]
+    w = np.arange(4)[None, None, None, :, None]
+    half = np.arange(2)[None, None, None, None, :]
+    k0 = 16 * kt + 2 * (th % 4)
+    nn = 64 * nt + 16 * w + th // 4 + 8 * half
+    for j, dk in enumerate((0, 8, 1, 9)):
+        kk, n2 = np.broadcast_arrays(k0 + dk, nn)
+        out[kk, n2] = (wa >> np.uint32(8 * j)) & 0xFF
+    return torch.from_numpy(out)
+
+
 def weight_perm_table(num_bits: int = 4) -> np.ndarray:
     """1024-entry permutation over a flattened [64 n-cols ... ] 16x64 tile, built from the
     thread/fragment description: 32 threads x 4 sub-tiles x 8 values, then the
@@ -95,18 +143,20 @@ def marlin_weights_perm_table(q, perm=None, num_bits: int = 4) -> torch.Tensor:
 
 
 def gptq_marlin_repack(b_q_weight, perm, size_k: int, size_n: int, num_bits: int = 4) -> torch.Tensor:
-    """GPTQ checkpoint int32 [K/8, N] (+ optional row order) -> Marlin int32 [K/16, 2N]."""
-    assert num_bits == 4
-    assert tuple(b_q_weight.shape) == (size_k // 8, size_n)
-    q = unpack_rows(b_q_weight, 4)
-    return marlin_weights_closed_form(q, perm if perm is not None and len(perm) else None)
+    """GPTQ checkpoint int32 [K/pf, N] (+ optional row order) -> Marlin int32 [K/16, N*16/pf], pf = 32/num_bits."""
+    assert num_bits in (4, 8)
+    assert tuple(b_q_weight.shape) == (size_k // (32 // num_bits), size_n)
+    q = unpack_rows(b_q_weight, num_bits)
+    p = perm if perm is not None and len(perm) else None
+    return marlin_weights_closed_form(q, p) if num_bits == 4 else marlin_weights_closed_form8(q, p)
 
 
 def awq_marlin_repack(b_q_weight, size_k: int, size_n: int, num_bits: int = 4) -> torch.Tensor:
-    """AWQ checkpoint int32 [K, N/8] -> Marlin int32 [K/16, 2N]."""
-    assert num_bits == 4
-    assert tuple(b_q_weight.shape) == (size_k, size_n // 8)
-    return marlin_weights_closed_form(awq_unpack(b_q_weight, 4))
+    """AWQ checkpoint int32 [K, N/pf] -> Marlin int32 [K/16, N*16/pf], pf = 32/num_bits."""
+    assert num_bits in (4, 8)
+    assert tuple(b_q_weight.shape) == (size_k, size_n // (32 // num_bits))
+    q = awq_unpack(b_q_weight, num_bits)
+    return marlin_weights_closed_form(q) if num_bits == 4 else marlin_weights_closed_form8(q)
 
 
 def marlin_unpack_weights(marlin_w) -> torch.Tensor:

@@ -27,14 +27,15 @@ class Layer:
     marlin_zp: torch.Tensor      # int32 [G, N/8] or empty
     g_idx_sorted: torch.Tensor   # int32 [K] or empty
     sort_indices: torch.Tensor   # int32 [K] or empty
+    bits: int = 4
 
     @property
     def type_id(self):
-        return (st.uint4 if self.has_zp else st.uint4b8).id
+        return (st.uint4 if self.has_zp else st.uint4b8 if self.bits == 4 else st.uint8b128).id
 
 
 def make_layer(size_k, size_n, group_size, dtype=torch.float16, has_zp=False, act_order=False, seed=0,
-               w_std=1.0, rule="reference") -> Layer:
+               w_std=1.0, rule="reference", bits=4) -> Layer:
     g = torch.Generator().manual_seed(seed)
     w = (torch.randn(size_k, size_n, generator=g) * w_std).to(dtype)
     empty_i = torch.empty(0, dtype=torch.int32)
@@ -51,7 +52,8 @@ def make_layer(size_k, size_n, group_size, dtype=torch.float16, has_zp=False, ac
                      ml.marlin_permute_scales(s, size_k, size_n, gs), marlin_zp, empty_i, empty_i)
     if rule == "reference":
         perm = torch.randperm(size_k, generator=g) if act_order else None
-        w_ref, q, s, g_idx, _ = qu.gptq_quantize_weights(w, st.uint4b8, group_size, act_order, perm)
+        w_ref, q, s, g_idx, _ = qu.gptq_quantize_weights(w, st.uint4b8 if bits == 4 else st.uint8b128, group_size,
+                                                         act_order, perm)
     else:
         assert not act_order
         w_ref, q, s = qu.quantize_absmax7(w, group_size)
@@ -59,15 +61,16 @@ def make_layer(size_k, size_n, group_size, dtype=torch.float16, has_zp=False, ac
     sort_indices, g_idx_sorted, q_sorted = empty_i, empty_i, q
     if act_order:
         q_sorted, g_idx_sorted, sort_indices = qu.sort_weights(q, g_idx)
-    marlin_q = ml.marlin_weights_closed_form(q_sorted)
+    marlin_q = ml.marlin_weights_closed_form(q_sorted) if bits == 4 else ml.marlin_weights_closed_form8(q_sorted)
     return Layer(size_k, size_n, group_size, dtype, False, act_order, w_ref, q, s, None, g_idx, marlin_q,
-                 ml.marlin_permute_scales(s, size_k, size_n, gs), empty_i, g_idx_sorted, sort_indices)
+                 ml.marlin_permute_scales(s, size_k, size_n, gs), empty_i, g_idx_sorted, sort_indices, bits)
 
 
 def run_gemm(ops, layer: Layer, a, dev, workspace, is_k_full=True, bias=None, use_atomic_add=False, c=None):
     """Call the op the way the reference's kernel test does (test_marlin_gemm.py:330-349)."""
     import vllm_amd.scalar_type as vst
-    wtype = vst.scalar_types.uint4 if layer.has_zp else vst.scalar_types.uint4b8
+    wtype = (vst.scalar_types.uint4 if layer.has_zp else
+             vst.scalar_types.uint4b8 if layer.bits == 4 else vst.scalar_types.uint8b128)
     return ops.gptq_marlin_gemm(
         a, c, layer.marlin_q.to(dev), None if bias is None else bias, layer.marlin_s.to(dev), None,
         layer.marlin_zp.to(dev), layer.g_idx_sorted.to(dev), layer.sort_indices.to(dev), workspace, wtype,

@@ -75,7 +75,7 @@ def test_kernel_selection_errors(dev):
     with pytest.raises(ValueError, match="min_thread_n"):
         choose_mp_linear_kernel(bad)
     bad8 = MPLinearLayerConfig(full_weight_shape=(1024, 128), partition_weight_shape=(1024, 128),
-                               weight_type=scalar_types.uint8b128, act_type=torch.float16, group_size=128,
+                               weight_type=scalar_types.int8, act_type=torch.float16, group_size=128,
                                zero_points=False, has_g_idx=False)
     with pytest.raises(ValueError, match="not supported"):
         choose_mp_linear_kernel(bad8)

@@ -1,0 +1,82 @@
+"""uint8b128 (W8A16) on the same operator surface: repack bit-exact, GEMM against the CPU oracle."""
+import pytest
+import torch
+
+from helpers import check_close, make_layer, run_gemm
+from oracle import marlin_layout as ml
+from oracle import quant_utils as qu
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import vllm_amd.ops as o
+    return o
+
+
+@pytest.fixture(scope="module")
+def workspace(dev):
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    return marlin_make_workspace_new(dev)
+
+
+@pytest.mark.parametrize("k,n", [(16, 64), (128, 192), (1024, 512)])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_repack8_bit_exact(ops, dev, k, n, act_order):
+    g = torch.Generator().manual_seed(k + n)
+    q = torch.randint(0, 256, (k, n), generator=g, dtype=torch.int32)
+    perm = torch.randperm(k, generator=g).to(torch.int32) if act_order else torch.empty(0, dtype=torch.int32)
+    got = ops.gptq_marlin_repack(qu.pack_rows(q, 8).to(dev), perm.to(dev), k, n, 8)
+    assert got.shape == (k // 16, 4 * n)
+    assert torch.equal(got.cpu(), ml.gptq_marlin_repack(qu.pack_rows(q, 8), perm, k, n, 8))
+    if not act_order:
+        got = ops.awq_marlin_repack(qu.awq_pack(q, 8).to(dev), k, n, 8)
+        assert torch.equal(got.cpu(), ml.marlin_weights_closed_form8(q))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 32, 128])
+def test_one_hot_rows_are_exact_w8(ops, dev, workspace, dtype, group):
+    k, n = 512, 192
+    layer = make_layer(k, n, group, dtype, seed=3, bits=8)
+    ks = torch.randperm(k, generator=torch.Generator().manual_seed(1))[:40]
+    a = torch.zeros(40, k, dtype=dtype)
+    a[torch.arange(40), ks] = 1.0
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 16, 33, 100, 512])
+@pytest.mark.parametrize("group,act_order,k_full", [(-1, False, True), (128, False, True), (64, True, True), (128, True, False)])
+def test_gemm_w8(ops, dev, workspace, dtype, m, group, act_order, k_full):
+    k, n = 1024, 384
+    layer = make_layer(k, n, group, dtype, act_order=act_order, seed=m + k, bits=8)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(2)).to(dtype).to(dev)
+    out = run_gemm(ops, layer, a, dev, workspace, is_k_full=k_full)
+    check_close(out, a, layer)
+    assert int(workspace.abs().sum()) == 0
+
+
+def test_linear_kernel_w8(dev):
+    from vllm_amd.mixed_precision import MarlinLinearKernel, MPLinearLayerConfig, choose_mp_linear_kernel
+    from vllm_amd.scalar_type import scalar_types
+    from oracle import gemm_ref as gr
+    from oracle import scalar_types as ost
+    k, n, m = 512, 256, 20
+    w = (torch.randn(k, n, generator=torch.Generator().manual_seed(0)) * 0.05).half()
+    w_ref, q, s, _, _ = qu.gptq_quantize_weights(w, ost.uint8b128, 128, False, None)
+    layer = torch.nn.Module()
+    layer.qweight = torch.nn.Parameter(qu.pack_rows(q, 8).to(dev), requires_grad=False)
+    layer.scales = torch.nn.Parameter(s.to(dev), requires_grad=False)
+    cfg = MPLinearLayerConfig(full_weight_shape=(k, n), partition_weight_shape=(k, n), weight_type=scalar_types.uint8b128,
+                              act_type=torch.float16, group_size=128, zero_points=False, has_g_idx=False)
+    assert choose_mp_linear_kernel(cfg) is MarlinLinearKernel
+    kern = MarlinLinearKernel(cfg, "qweight", "scales")
+    kern.process_weights_after_loading(layer)
+    assert tuple(layer.qweight.shape) == (k // 16, 4 * n)
+    x = torch.randn(m, k, generator=torch.Generator().manual_seed(1)).half()
+    out = kern.apply_weights(layer, x.to(dev))
+    mt = gr.error_metrics(out, gr.gemm_ref(x, w_ref))
+    assert mt["max_rel"] <= 2e-2 and mt["mean_rel"] < 0.04, mt

@@ -141,3 +141,42 @@ def test_zero_points_closed_form_and_known_word():
     assert torch.equal(a, ml.marlin_zero_points_closed_form(z))
     assert torch.equal(ml.marlin_unpack_zero_points(a), z)
     assert torch.equal(ml.awq_to_marlin_zero_points(qu.awq_pack(z), 3, 192), a)
+
+
+# ------------------------------------------------------------------------------ 8-bit weights
+def rand_q8(k, n, seed=0):
+    return torch.randint(0, 256, (k, n), generator=torch.Generator().manual_seed(seed), dtype=torch.int32)
+
+
+def test_weights8_known_words():
+    """q[k,n] = k: word th*8 + 2w + half holds rows r, r+8, r+1, r+9 (r = 2(th%4)) in bytes 0..3."""
+    q = torch.arange(16, dtype=torch.int32).view(16, 1).expand(16, 64).contiguous()
+    w = u32(ml.marlin_weights_closed_form8(q))[0]
+    assert [hex(int(w[8 * th])) for th in range(4)] == ["0x9010800", "0xb030a02", "0xd050c04", "0xf070e06"]
+    # q[k,n] = n: every byte of word (th, w, half) is the column 16w + th//4 + 8*half
+    q = torch.arange(64, dtype=torch.int32).view(1, 64).expand(16, 64).contiguous()
+    w = u32(ml.marlin_weights_closed_form8(q))[0]
+    for th, sub, half in ((0, 0, 0), (5, 1, 1), (31, 3, 1)):
+        col = 16 * sub + th // 4 + 8 * half
+        assert int(w[th * 8 + 2 * sub + half]) == col * 0x01010101
+
+
+@pytest.mark.parametrize("k,n", [(16, 64), (64, 192)])
+def test_weights8_two_formulations_inverse_and_checkpoints(k, n):
+    q = rand_q8(k, n, seed=k * n)
+    a = ml.marlin_weights_closed_form8(q)
+    assert a.shape == (k // 16, 4 * n)
+    assert torch.equal(a, ml.marlin_weights_perm_table(q, num_bits=8))
+    assert torch.equal(ml.marlin_unpack_weights8(a), q)
+    assert torch.equal(ml.gptq_marlin_repack(qu.pack_rows(q, 8), None, k, n, 8), a)
+    assert torch.equal(ml.awq_marlin_repack(qu.awq_pack(q, 8), k, n, 8), a)
+    perm = torch.randperm(k, generator=torch.Generator().manual_seed(2)).to(torch.int32)
+    assert torch.equal(ml.gptq_marlin_repack(qu.pack_rows(q, 8), perm, k, n, 8), ml.marlin_weights_closed_form8(q[perm.long()]))
+
+
+def test_pack8_literals():
+    q = torch.tensor([[1], [2], [3], [4]], dtype=torch.int32)
+    assert int(u32(qu.pack_rows(q, 8))[0, 0]) == 0x04030201
+    q = torch.tensor([[1, 2, 3, 4]], dtype=torch.int32)
+    assert int(u32(qu.awq_pack(q, 8))[0, 0]) == 0x04020301      # byte t holds column (0, 2, 1, 3)[t]
+    assert torch.equal(qu.awq_unpack(qu.awq_pack(q, 8), 8), q)

@@ -161,3 +161,21 @@ def test_gemm_ref_is_fp32_matmul_plus_bias():
     assert out.tolist() == [[5.0, 7.0], [1.0, -5.0]]
     m = gr.error_metrics(out + torch.tensor([[0.0, 0.7], [0.0, 0.0]]), out)
     assert abs(m["max_rel"] - 0.1) < 1e-6 and abs(m["mean_rel"] - 0.7 / 18.0) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 128])
+def test_uint8b128_quantizer_and_dequant(dtype, group):
+    k, n = 256, 64
+    w = torch.randn(k, n, generator=torch.Generator().manual_seed(6)).to(dtype)
+    w_ref, q, s, zp = qu.quantize_weights(w, st.uint8b128, group)
+    assert zp is None and q.min() >= 0 and q.max() <= 255
+    gs = k if group == -1 else group
+    assert torch.equal(w_ref, (q - 128).to(dtype) * s.repeat_interleave(gs, 0))
+    mq = ml.gptq_marlin_repack(qu.pack_rows(q, 8), None, k, n, 8)
+    ms = ml.marlin_permute_scales(s, k, n, gs)
+    assert torch.equal(gr.dequant_marlin(mq, ms, None, None, k, n, True, dtype, num_bits=8), w_ref)
+    # symmetric rule: s = max(|max| / 127, |min| / 128)
+    wg = w.float().view(k // gs, gs, n)
+    want = torch.maximum(wg.amax(1).abs() / 127, wg.amin(1).abs() / 128)
+    assert torch.allclose(s.float(), want, rtol=2e-2)

@@ -85,12 +85,19 @@ def _wtype_code(type_id: int, has_zp: bool) -> int:
     if type_id == scalar_types.uint4b8.id:
         _check(not has_zp, "b_q_type must be uint4 or uint8 when has_zp = True. Got = uint4b8")
         return _lib.WTYPE_U4B8
+    if type_id == scalar_types.uint8b128.id:
+        _check(not has_zp, "b_q_type must be uint4 or uint8 when has_zp = True. Got = uint8b128")
+        return _lib.WTYPE_U8B128
     if type_id == scalar_types.uint4.id:
         _check(has_zp, "b_q_type must be uint4b8 or uint8b128 when has_zp = False. Got = uint4")
         return _lib.WTYPE_U4
     raise NotImplementedError(
         f"weight type {ScalarType.from_id(type_id)} is not implemented by the gfx950 W4A16 library "
-        "(supported: uint4b8, uint4 with zero points)")
+        "(supported: uint4b8, uint8b128, uint4 with zero points)")
+
+
+def _pack_factor(type_id: int) -> int:
+    return 32 // ScalarType.from_id(int(type_id)).size_bits
 
 
 # ------------------------------------------------------------------------------- implementations
@@ -191,8 +198,9 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
     _check(b_q_weight.dim() == 2 and size_k // 16 == b_q_weight.size(0),
            f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, tile_size = 16")
     _check(b_q_weight.size(1) % 16 == 0, f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = 16")
-    _check(size_n == b_q_weight.size(1) // 16 * 8,
-           f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_n = {size_n}, pack_factor = 8")
+    pf = _pack_factor(b_q_type)
+    _check(size_n == b_q_weight.size(1) // 16 * pf,
+           f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_n = {size_n}, pack_factor = {pf}")
     _check(a.is_cuda, "A is not on GPU")
     _check(a.stride(1) == 1, "A.stride(1) is not 1")
     _check(a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8")
@@ -268,8 +276,9 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
     num_experts = b_q_weight.size(0)
     _check(size_k % 16 == 0 and b_q_weight.size(1) == size_k // 16,
            f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_k = {size_k}, tile_size = 16")
-    _check(b_q_weight.size(2) % 16 == 0 and size_n == b_q_weight.size(2) // 16 * 8,
-           f"Shape mismatch: b_q_weight.size(2) = {b_q_weight.size(2)}, size_n = {size_n}, pack_factor = 8")
+    pf = _pack_factor(b_q_type_id)
+    _check(b_q_weight.size(2) % 16 == 0 and size_n == b_q_weight.size(2) // 16 * pf,
+           f"Shape mismatch: b_q_weight.size(2) = {b_q_weight.size(2)}, size_n = {size_n}, pack_factor = {pf}")
     _check(b_scales.is_cuda and b_scales.is_contiguous() and b_scales.dim() == 3, "b_scales rank is not 3")
     _check(b_scales.size(0) == num_experts and b_scales.size(2) == size_n and b_scales.dtype == a.dtype,
            f"b_scales dim 2 = {b_scales.size(2)} is not size_n = {size_n}")

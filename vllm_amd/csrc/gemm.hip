@@ -18,7 +18,8 @@ static int validate(const w4a16_gemm_args* a) {
               a->struct_size, sizeof(w4a16_gemm_args));
   W4A16_CHECK(a->dtype == W4A16_DTYPE_F16 || a->dtype == W4A16_DTYPE_BF16,
               "gpt_marlin_gemm only supports bfloat16 and float16");
-  W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U4, "unsupported b_q_type");
+  W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U4 || a->wtype == W4A16_WTYPE_U8B128,
+              "unsupported b_q_type");
   W4A16_CHECK(a->size_m >= 0 && a->size_n > 0 && a->size_k > 0, "bad problem size");
   W4A16_CHECK(a->size_k % 32 == 0, "size_k = %lld is not divisible by 32", (long long)a->size_k);
   W4A16_CHECK(a->size_n % 64 == 0, "size_n = %lld is not divisible by tile_n_size = 64", (long long)a->size_n);
@@ -33,7 +34,8 @@ static int validate(const w4a16_gemm_args* a) {
   if (has_zp)
     W4A16_CHECK(a->wtype == W4A16_WTYPE_U4, "b_q_type must be uint4 when has_zp = True");
   else
-    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8, "b_q_type must be uint4b8 when has_zp = False");
+    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U8B128,
+                "b_q_type must be uint4b8 or uint8b128 when has_zp = False");
   W4A16_CHECK((a->g_idx == nullptr) == (a->perm == nullptr),
               "g_idx and perm must both be given (act-order) or both be empty");
   if (a->flags & W4A16_F_MOE) {
@@ -70,6 +72,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
 
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
+  const bool w8 = a->wtype == W4A16_WTYPE_U8B128;  // 8-bit weights: general kernel only
+  if (w8 && moe && act_order)
+    return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
   if (moe) {
     const int bs = a->moe_block_size;
     pl.mb = bs <= 16 ? 1 : bs <= 32 ? 2 : 4;
@@ -95,7 +100,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
-  if (!moe && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  if (!moe && !w8 && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
@@ -118,7 +123,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   {
     const int64_t mid_mtiles = moe ? ceil_div(a->n_sorted, 64) : ceil_div(a->size_m, 64);
     const int64_t mid_tiles = mid_mtiles * ceil_div(a->size_n, 512);
-    const bool mid_shape = a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+    const bool mid_shape = !w8 && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
                            (moe ? a->moe_block_size == 64 : (a->size_m > 32 && mid_tiles >= cus / 2));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
       W4A16_CHECK(mid_tiles < (1LL << 31) / 64, "too many tiles");
@@ -138,7 +143,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
 
   // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
-  const bool decode_shape = pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
+  const bool decode_shape = !w8 && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
                             (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
 
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these

@@ -193,6 +193,40 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t xa, uint32_t xb, cons
   }
 }
 
+// 8-bit weights (uint8b128: stored byte = value + 128).  A lane's Marlin word holds the bytes of one column for
+// K rows (k0, k0+8, k0+1, k0+9); ha / hb: the words of column half 0 / half 1, a / b: k-tiles 2ks / 2ks+1.
+//  fp16:  (1024 + b) - 1152 is exact, then one multiply by s (= half(q - 128) * half(s), the reference's w_ref)
+//  bf16:  bf16_rne(fma(float(b), s, -128 s))
+template <int DT, bool UNIT_SCALE>
+__device__ __forceinline__ void dequant_pair8(uint32_t xa0, uint32_t xa1, uint32_t xb0, uint32_t xb1,
+                                              uint32_t s_pair, u32x4& o0, u32x4& o1) {
+  if constexpr (DT == DT_F16) {
+    uint32_t EX = 0x64006400u;
+    asm("" : "+v"(EX));
+    const f16x2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const f16x2 s = as_h2(s_pair);
+    auto lo = [&](uint32_t x, f16x2 sc) {
+      const f16x2 v = as_h2((x & 0x00ff00ffu) | EX) - bias;
+      return as_u32(UNIT_SCALE ? v : v * sc);
+    };
+    auto hi = [&](uint32_t x, f16x2 sc) { return lo(x >> 8, sc); };
+    const f16x2 s0 = {s.x, s.x}, s1 = {s.y, s.y};
+    o0 = u32x4{lo(xa0, s0), hi(xa0, s0), lo(xb0, s0), hi(xb0, s0)};
+    o1 = u32x4{lo(xa1, s1), hi(xa1, s1), lo(xb1, s1), hi(xb1, s1)};
+  } else {
+    const float s0 = UNIT_SCALE ? 1.0f : bf16_lo_f32(s_pair), s1 = UNIT_SCALE ? 1.0f : bf16_hi_f32(s_pair);
+    const float c0 = -128.0f * s0, c1 = -128.0f * s1;
+    auto lo = [&](uint32_t x, float sf, float cf) {
+      return pack_bf16(__builtin_fmaf(ubyte_f32<0>(x), sf, cf), __builtin_fmaf(ubyte_f32<2>(x), sf, cf));
+    };
+    auto hi = [&](uint32_t x, float sf, float cf) {
+      return pack_bf16(__builtin_fmaf(ubyte_f32<1>(x), sf, cf), __builtin_fmaf(ubyte_f32<3>(x), sf, cf));
+    };
+    o0 = u32x4{lo(xa0, s0, c0), hi(xa0, s0, c0), lo(xb0, s0, c0), hi(xb0, s0, c0)};
+    o1 = u32x4{lo(xa1, s1, c1), hi(xa1, s1, c1), lo(xb1, s1, c1), hi(xb1, s1, c1)};
+  }
+}
+
 // "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
 // of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
 // high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the

@@ -1,4 +1,4 @@
-// W4A16 "skinny" GEMM for gfx950: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias), dense or fused-MoE.
+// W4A16 (and W8A16, uint8b128) "skinny" GEMM for gfx950: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias), dense or fused-MoE.
 //
 // Stands in for the reference's Marlin<> kernel (csrc/quantization/gptq_marlin/marlin_template.h:273-1804)
 // and its MoE twin (csrc/moe/marlin_moe_wna16/marlin_template.h:298-2009); written from scratch for
@@ -12,8 +12,8 @@
 //   wavefront waits on another inside the main loop:
 //     weights      global -> registers, 128-bit per lane, 1 KiB contiguous per wavefront instruction,
 //                  D k-steps (2D KiB) in flight per wavefront
-//     activations  global -> registers, 16 bytes per lane (row l&15, 8 consecutive K), turned into the
-//                  MFMA A operand by a 4x4 lane-group/register transpose (4 v_permlane*_swap); no LDS
+//     activations  global -> registers, 16 bytes per lane (coalesced rows), bounced through a
+//                  wavefront-private LDS slab into the MFMA A operand order (no barrier needed)
 //     scales/zeros one 16-byte / 4-byte load per k-step (cache hits after the first of a group)
 //   The 8 partial tiles are summed through LDS.  Splits are summed by the last workgroup to arrive
 //   at the tile's counter in `workspace`, in split order (deterministic); the counter is reset so
@@ -23,6 +23,7 @@
 #include <stdlib.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "gemm_kernels.h"
 
@@ -37,14 +38,16 @@ struct SkinnyCfg {
 };
 
 
-template <int DT, int MB, bool ZP, int GM, bool PERM>
+template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
+  static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
   constexpr int BM = 16 * MB;
-  constexpr int D = SkinnyCfg<MB>::D;
+  // 8-bit stages hold twice the weight registers: shorter ring
+  constexpr int D = (BITS == 8) ? (MB >= 4 ? 2 : 3) : SkinnyCfg<MB>::D;
   constexpr bool UNIT = (GM == GM_CHANNEL);
   // Decode tiles (one m-block) keep the weights as raw magic numbers E+q in the MFMA and apply
   // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
-  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX);
+  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4);
   constexpr bool HI_TRICK = FOLD && (DT == DT_F16) && !ZP;
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
@@ -134,8 +137,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 
   // lanes of an n-tile past the end of N (odd number of n-tiles) read n-tile 0; their columns are never stored
   const int nt = (2 * cp + h) * 64 < p.N ? 2 * cp + h : 0;
-  const int64_t b_row = p.N >> 1;  // u32x4 per k-tile row
-  const u32x4* bp = (const u32x4*)Bq + nt * 32 + (4 * c + g);
+  // 4-bit: 32 u32x4 per n-tile and k-tile, one per Marlin thread; 8-bit: 64, two per thread (words 2w + half)
+  const int64_t b_row = (BITS == 4) ? (p.N >> 1) : p.N;  // u32x4 per k-tile row
+  const u32x4* bp = (const u32x4*)Bq + nt * (8 * BITS) + (4 * c + g) * (BITS / 4);
   const int64_t s_row = p.N >> 3;  // u32x4 (8 scales) per scale row; also words per zero-point row
   const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
@@ -151,6 +155,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
   struct Stage {
     u32x4 b0, b1, sc;
+    u32x4 b0h, b1h;  // 8-bit weights only: second half of the thread's words (w = 2, 3)
     u32x4 a[MB];
     uint32_t zq;
     int gi;
@@ -184,6 +189,29 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     s.b0 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks) * b_row);
     s.b1 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks + 1) * b_row);
+    if constexpr (BITS == 8) {
+      s.b0h = __builtin_nontemporal_load(bp + (int64_t)(2 * ks) * b_row + 1);
+      s.b1h = __builtin_nontemporal_load(bp + (int64_t)(2 * ks + 1) * b_row + 1);
+    }
+  };
+  // B operands (column half 0 / 1) of Marlin word position w of a stage; unit: leave the scale out
+  auto dequant_word = [&](const Stage& s, auto w_tag, auto unit_tag, u32x4& o0, u32x4& o1) {
+    constexpr int w = decltype(w_tag)::value;
+    constexpr bool unit = decltype(unit_tag)::value;
+    if constexpr (BITS == 4) {
+      uint32_t z0 = 8, z1 = 8;
+      if (ZP) {
+        z0 = (s.zq >> (4 * w)) & 0xf;
+        z1 = (s.zq >> (4 * w + 16)) & 0xf;
+      }
+      const ColConst<DT> cc = make_col_const<DT, unit>(unit ? 0u : s.sc[w], z0, z1);
+      dequant_pair<DT, unit>(s.b0[w], s.b1[w], cc, o0, o1);
+    } else {
+      const u32x4& la = (w < 2) ? s.b0 : s.b0h;
+      const u32x4& lb = (w < 2) ? s.b1 : s.b1h;
+      dequant_pair8<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
+                              unit ? 0u : s.sc[w], o0, o1);
+    }
   };
 
   f32x4 acc[MB][4][2];
@@ -289,11 +317,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
         const int kk = kb + (e & 1) + ((e >> 1) & 1) * 8 + (e >> 2) * 16;
         se[e] = sp[(int64_t)gidx[kk] * s_row];
       }
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const ColConst<DT> cc = make_col_const<DT, true>(0, 8, 8);
+      auto gidx_word = [&](auto w_tag) {
+        constexpr int w = decltype(w_tag)::value;
         u32x4 o[2];
-        dequant_pair<DT, true>(s.b0[w], s.b1[w], cc, o[0], o[1]);
+        dequant_word(s, w_tag, std::true_type{}, o[0], o[1]);
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
           u32x4 r;
@@ -311,25 +338,27 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) acc[mb][w][hf] = mfma16x16x32<DT>(af[mb], r, acc[mb][w][hf]);
         }
-      }
+      };
+      gidx_word(std::integral_constant<int, 0>{});
+      gidx_word(std::integral_constant<int, 1>{});
+      gidx_word(std::integral_constant<int, 2>{});
+      gidx_word(std::integral_constant<int, 3>{});
       return;
     }
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t z0 = 8, z1 = 8;
-      if (ZP) {
-        z0 = (s.zq >> (4 * w)) & 0xf;
-        z1 = (s.zq >> (4 * w + 16)) & 0xf;
-      }
-      const ColConst<DT> cc = make_col_const<DT, UNIT>(GM == GM_CHANNEL ? 0u : s.sc[w], z0, z1);
+    auto plain_word = [&](auto w_tag) {
+      constexpr int w = decltype(w_tag)::value;
       u32x4 o0, o1;
-      dequant_pair<DT, UNIT>(s.b0[w], s.b1[w], cc, o0, o1);
+      dequant_word(s, w_tag, std::integral_constant<bool, UNIT>{}, o0, o1);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         acc[mb][w][0] = mfma16x16x32<DT>(af[mb], o0, acc[mb][w][0]);
         acc[mb][w][1] = mfma16x16x32<DT>(af[mb], o1, acc[mb][w][1]);
       }
-    }
+    };
+    plain_word(std::integral_constant<int, 0>{});
+    plain_word(std::integral_constant<int, 1>{});
+    plain_word(std::integral_constant<int, 2>{});
+    plain_word(std::integral_constant<int, 3>{});
   };
 
   // ---- software pipeline: D k-steps in flight.  The steady-state loop is free of conditionals so
@@ -490,7 +519,29 @@ static skinny_fn pick_mb(int mb, bool zp, int gm) {
   }
 }
 
-static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool perm) {
+template <int DT>
+static skinny_fn pick_w8(int mb, int gm) {  // uint8b128: no zero points, A's columns already in weight order
+  switch (mb) {
+    case 1:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, false, 8>
+             : gm == GM_CHANNEL ? skinny_kernel<DT, 1, false, GM_CHANNEL, false, 8>
+                                : skinny_kernel<DT, 1, false, GM_GIDX, false, 8>;
+    case 2:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, false, 8>
+             : gm == GM_CHANNEL ? skinny_kernel<DT, 2, false, GM_CHANNEL, false, 8>
+                                : skinny_kernel<DT, 2, false, GM_GIDX, false, 8>;
+    default:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, false, 8>
+             : gm == GM_CHANNEL ? skinny_kernel<DT, 4, false, GM_CHANNEL, false, 8>
+                                : skinny_kernel<DT, 4, false, GM_GIDX, false, 8>;
+  }
+}
+
+static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool perm, bool w8) {
+  if (w8) {
+    if (zp || perm) return nullptr;
+    return dt == DT_F16 ? pick_w8<DT_F16>(mb, gm) : pick_w8<DT_BF16>(mb, gm);
+  }
   if (perm) return dt == DT_F16 ? pick_mb<DT_F16, true>(mb, zp, gm) : pick_mb<DT_BF16, true>(mb, zp, gm);
   return dt == DT_F16 ? pick_mb<DT_F16, false>(mb, zp, gm) : pick_mb<DT_BF16, false>(mb, zp, gm);
 }
@@ -501,7 +552,7 @@ static int skinny_smem_bytes(int mb) {
 
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
-  skinny_fn fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm);
+  skinny_fn fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
   if (!fn) return fail(W4A16_EINVAL, "unsupported kernel variant");
   KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);

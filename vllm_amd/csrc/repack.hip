@@ -1,4 +1,4 @@
-// Checkpoint -> Marlin-layout repack kernels (4-bit), written for gfx950.
+// Checkpoint -> Marlin-layout repack kernels (4-bit, and a simple 8-bit variant), written for gfx950.
 //
 // Output layout (int32 [K/16, 2N]): for k-tile kt (16 rows) and n-tile nt (64 cols) the 128
 // words nt*128 + th*4 + w (th in [0,32), w in [0,4)) hold, with r = 2*(th%4), c = th/4,
@@ -109,6 +109,41 @@ __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restr
   out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
 }
 
+// 8-bit variant (uint8b128): output int32 [K/16, 4N]; per k-tile and n-tile 256 words; word
+// nt*256 + th*8 + 2w + half holds the bytes q[k0 + {0, 8, 1, 9}[j], 64nt + 16w + c + 8 half], j = 0..3
+// (gptq_marlin_repack.cu:119-203 with num_bits = 8).  One thread per output word; load-time only, so the
+// gathers are not staged.  GPTQ source: word (r, n), byte i = q[4r + i, n]; AWQ source: word (k, cw),
+// byte t = q[k, 4cw + {0, 2, 1, 3}[t]].
+template <bool AWQ, bool HAS_PERM>
+__global__ __launch_bounds__(256) void repack8_kernel(const uint32_t* __restrict__ in, const int32_t* __restrict__ perm,
+                                                      uint32_t* __restrict__ out, int size_k, int size_n) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // output word
+  const int64_t row_words = 4LL * size_n;
+  if (idx >= (int64_t)(size_k / 16) * row_words) return;
+  const int kt = (int)(idx / row_words);
+  const int rem = (int)(idx % row_words);
+  const int nt = rem >> 8, th = (rem >> 3) & 31, w = (rem >> 1) & 3, half = rem & 1;
+  const int k0 = 16 * kt + 2 * (th & 3);
+  const int n = 64 * nt + 16 * w + (th >> 2) + 8 * half;
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int k = k0 + ((j & 1) ? 8 : 0) + (j >> 1);  // {0, 8, 1, 9}[j]
+    if (HAS_PERM) k = perm[k];
+    uint32_t b;
+    if (AWQ) {
+      const uint32_t src = in[(size_t)k * (size_n >> 2) + (n >> 2)];
+      const int pos = ((n & 1) << 1) | ((n >> 1) & 1);  // {0, 2, 1, 3}[n % 4]
+      b = (src >> (8 * pos)) & 0xFFu;
+    } else {
+      const uint32_t src = in[(size_t)(k >> 2) * size_n + n];
+      b = (src >> (8 * (k & 3))) & 0xFFu;
+    }
+    word |= b << (8 * j);
+  }
+  out[idx] = word;
+}
+
 // out[m, k] = a[m, perm[k]], 16-bit elements.
 __global__ __launch_bounds__(256) void permute_cols_kernel(const uint16_t* __restrict__ a,
                                                            const int32_t* __restrict__ perm,
@@ -123,8 +158,8 @@ static int check_repack(int64_t size_k, int64_t size_n, int num_bits) {
   W4A16_CHECK(size_k % 16 == 0, "size_k = %lld is not divisible by tile_k_size = 16", (long long)size_k);
   W4A16_CHECK(size_n % 64 == 0, "size_n = %lld is not divisible by tile_n_size = 64", (long long)size_n);
   W4A16_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = %d", num_bits);
-  if (num_bits == 8) return fail(W4A16_ENOTIMPL, "8-bit Marlin repack is not implemented in this build");
   W4A16_CHECK(size_k / 16 <= 65535, "size_k = %lld too large", (long long)size_k);
+  W4A16_CHECK(size_k / 16 * 4 * size_n < (1LL << 31) * 256, "problem too large");
   return 0;
 }
 
@@ -137,8 +172,17 @@ extern "C" int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
   if (int rc = check_repack(size_k, size_n, num_bits)) return rc;
   W4A16_CHECK(b_q_weight && out, "null weight pointer");
   if (size_k == 0 || size_n == 0) return 0;
-  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
   hipStream_t s = (hipStream_t)stream;
+  if (num_bits == 8) {
+    const unsigned blocks = (unsigned)ceil_div(size_k / 16 * 4 * size_n, 256);
+    if (perm)
+      repack8_kernel<false, true><<<blocks, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n);
+    else
+      repack8_kernel<false, false><<<blocks, 256, 0, s>>>(b_q_weight, nullptr, out, (int)size_k, (int)size_n);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
+  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
   if (perm)
     gptq_repack_kernel<true><<<grid, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n);
   else
@@ -152,6 +196,12 @@ extern "C" int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out
   if (int rc = check_repack(size_k, size_n, num_bits)) return rc;
   W4A16_CHECK(b_q_weight && out, "null weight pointer");
   if (size_k == 0 || size_n == 0) return 0;
+  if (num_bits == 8) {
+    const unsigned blocks = (unsigned)ceil_div(size_k / 16 * 4 * size_n, 256);
+    repack8_kernel<true, false><<<blocks, 256, 0, (hipStream_t)stream>>>(b_q_weight, nullptr, out, (int)size_k, (int)size_n);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
   dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
   awq_repack_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k, (int)size_n);
   W4A16_HIP(hipGetLastError());

@@ -81,8 +81,9 @@ def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, ga
     if inplace:
         assert output is None, "Conflicting request"
     quant_type = ScalarType.from_id(quant_type_id)
-    assert quant_type in (scalar_types.uint4, scalar_types.uint4b8), f"unsupported MoE weight type {quant_type}"
-    num_bits = 4
+    assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128), \
+        f"unsupported MoE weight type {quant_type}"
+    num_bits = quant_type.size_bits
     M, K = hidden_states.size()
     E = w1.size(0)
     topk = topk_ids.size(1)

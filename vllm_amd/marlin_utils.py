@@ -23,11 +23,11 @@ _INTERLEAVE_4BIT = (0, 2, 4, 6, 1, 3, 5, 7)
 
 def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True,
                                        device_capability: int | None = None) -> list[ScalarType]:
-    """marlin_utils.py:35-78, narrowed to the types this library implements (4-bit)."""
+    """marlin_utils.py:35-78, narrowed to the types this library implements."""
     if has_zp is None:
         return (query_marlin_supported_quant_types(False, include_fp_type, device_capability) +
                 query_marlin_supported_quant_types(True, include_fp_type, device_capability))
-    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8]
+    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8, scalar_types.uint8b128]
 
 
 def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,

@@ -4,8 +4,8 @@ Mirrors vllm/model_executor/layers/quantization/kernels/mixed_precision/MPLinear
 (MPLinearLayerConfig, MPLinearKernel) and .../mixed_precision/marlin.py:28-166 (MarlinLinearKernel):
 same constructor, same `can_implement / process_weights_after_loading / apply_weights` contract,
 same parameter names left on the layer, so a vLLM LinearMethod can hold either class.
-Differences: `can_implement` accepts a ROCm gfx950 device instead of requiring CUDA, and only the
-4-bit types (uint4b8, uint4 + zero points) are offered.
+Differences: `can_implement` accepts a ROCm gfx950 device instead of requiring CUDA, and the types offered
+are uint4b8, uint8b128 and uint4 + zero points.
 """
 from abc import ABC, abstractmethod
 from collections.abc import Callable
