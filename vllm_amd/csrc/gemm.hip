@@ -92,6 +92,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   static const int forced_splits = env_int("W4A16_SPLITS", 0);
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
+  static const int debug_plan = env_int("W4A16_DEBUG", 0);
 
   // Dense act-order: A's columns are gathered once into a_tmp by permute_cols (as the reference's
   // permute_cols_kernel, csrc/quantization/gptq_marlin/gptq_marlin.cu:68-120), so the GEMM kernels read A with
@@ -118,15 +119,30 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     return 0;
   }
 
-  // 64-row kernel: MoE blocks of 64 slots, and dense problems with too few rows or tiles for the prefill kernel
-  // but enough 64 x 512 tiles to occupy the chip without splitting K.
+  // 64-row kernel: MoE blocks of 64 slots, and dense problems with too few rows or tiles for the prefill kernel.
+  // It holds two workgroups per compute unit; with fewer tiles than that, K is split (>= 32 k-steps per split, in
+  // multiples of 4) and a second small kernel adds the partial tiles (~2 us launch + the partials' traffic).
   {
     const int64_t mid_mtiles = moe ? ceil_div(a->n_sorted, 64) : ceil_div(a->size_m, 64);
     const int64_t mid_tiles = mid_mtiles * ceil_div(a->size_n, 512);
+    int sp = 1;
+    // (measured: worth it from about cus/2 tiles up to 3/4 cus dense, up to cus for MoE, whose tile count is an upper bound)
+    if (mid_tiles >= cus / 2 && mid_tiles < (moe ? cus : cus * 3 / 4)) {
+      const int by_k = pl.total_ksteps / 32;
+      const int by_cus = (int)(2 * cus / mid_tiles);
+      sp = by_k < by_cus ? by_k : by_cus;
+      if (sp < 1) sp = 1;
+      if (sp > 16) sp = 16;
+    }
+    if (forced_splits > 0) sp = forced_splits;
+    int kps = (int)ceil_div(pl.total_ksteps, sp);
+    kps = (kps + 3) / 4 * 4;
+    sp = (int)ceil_div(pl.total_ksteps, kps);
     const bool mid_shape = !w8 && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
-                           (moe ? a->moe_block_size == 64 : (a->size_m > 32 && mid_tiles >= cus / 2));
+                           (moe ? a->moe_block_size == 64
+                                : (a->size_m > 32 && mid_tiles >= cus / 2));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
-      W4A16_CHECK(mid_tiles < (1LL << 31) / 64, "too many tiles");
+      W4A16_CHECK(mid_tiles * sp < (1LL << 31) / 64, "too many tiles");
       pl.kind = 3;
       pl.tn = 512;
       pl.mb = 4;
@@ -134,10 +150,13 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       pl.mtiles = (int)mid_mtiles;
       pl.ncp = (int)ceil_div(a->size_n, 512);
       pl.tiles = (int)mid_tiles;
-      pl.splits = 1;
-      pl.kps = pl.total_ksteps;
+      pl.splits = sp;
+      pl.kps = kps;
       pl.xcd_map = 0;
-      pl.ctmp_bytes = 0;
+      pl.ctmp_bytes = sp > 1 ? mid_tiles * sp * 64 * 512 * 4 : 0;
+      if (debug_plan)
+        fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=3 tiles=%d splits=%d kps=%d\n", (long long)a->size_m,
+                (long long)a->size_n, (long long)a->size_k, pl.tiles, pl.splits, pl.kps);
       return 0;
     }
   }
@@ -208,8 +227,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = kps;
     pl.splits = (int)ceil_div(pl.total_ksteps, kps);
   }
-  static const int debug = env_int("W4A16_DEBUG", 0);
-  if (debug)
+  if (debug_plan)
     fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=%d tn=%d mb=%d tiles=%d splits=%d kps=%d model_us=%.2f\n",
             (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, pl.kind, pl.tn, pl.mb, pl.tiles,
             pl.splits, pl.kps, best.t);

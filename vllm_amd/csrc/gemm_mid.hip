@@ -12,6 +12,11 @@
 //   activations  the workgroup stages 64 rows x 64 K (two k-steps) into LDS, double buffered, in MFMA fragment
 //                order (one conflict-free ds_read_b128 per operand); MoE rows are gathered through sorted_token_ids
 //                while staging.  One barrier per two k-steps.
+//   split-K      with too few tiles to fill the chip, K is cut into splits of whole loop iterations (multiples of
+//                128 K rows); each workgroup writes its fp32 partial tile to scratch with plain 128-bit stores and
+//                mid_reduce_kernel, launched right behind, adds the splits in order and finishes the rows.  (Passing
+//                128 KB partial tiles between running workgroups through device-coherent 8-byte accesses, as the
+//                16-row kernels do with their 4 KB tiles, was measured slower than not splitting at all.)
 // Requirements (host-checked): K % 128 == 0, scales grouped or channelwise (no per-row g_idx), A's columns already
 // in weight order (dense act-order is gathered beforehand), MoE block size 64.
 #include <type_traits>
@@ -40,7 +45,9 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
   // (MoE: neighbouring blocks mostly belong to the same expert)
   const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
-  const int mt = blockIdx.x % mtiles, nt4 = blockIdx.x / mtiles;
+  const int mt = blockIdx.x % mtiles;
+  const int split = (blockIdx.x / mtiles) % p.splits, nt4 = blockIdx.x / (mtiles * p.splits);
+  const int tile = nt4 * mtiles + mt;          // index of the output tile (partials)
   const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
   const int row0 = mt * MD_BM;
@@ -105,10 +112,13 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     a_wr[i] = (((piece >> 2) * MD_MB + (r >> 4)) * 64 + (r & 15)) * 4 + (piece & 3);
   }
   u32x4 areg[2];
+  // this workgroup's k-steps: [ks_b, ks_e), a multiple of 4 long (the host splits K in multiples of 4 k-steps)
+  const int ks_b = split * p.ksteps_per_split;
+  const int ks_e = min(ks_b + p.ksteps_per_split, p.total_ksteps);
   // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
   //  keeps the main loop free of branches)
-  auto load_a = [&](int chunk) {
-    chunk = min(chunk, p.total_ksteps / 2 - 1);
+  auto load_a = [&](int chunk) {  // chunk: relative to ks_b
+    chunk = min(ks_b / 2 + chunk, ks_e / 2 - 1);
 #pragma unroll
     for (int i = 0; i < 2; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
   };
@@ -126,8 +136,8 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     uint32_t zq;
   };
   Stage st[MD_D];
-  auto issue = [&](Stage& s, int ks) {
-    ks = min(ks, p.total_ksteps - 1);
+  auto issue = [&](Stage& s, int ks) {  // ks: relative to ks_b
+    ks = min(ks_b + ks, ks_e - 1);
     int gi = 0;
     if (!CHANNEL) gi = ks / p.group_ksteps;
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
@@ -153,7 +163,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       acc[mb][w][1] = f32x4{0, 0, 0, 0};
     }
 
-  const int nchunks = p.total_ksteps / 2;  // total_ksteps is a multiple of 4 (K % 128 == 0)
+  const int nchunks = (ks_e - ks_b) / 2;  // even: K % 128 == 0 and splits are multiples of 4 k-steps
 
   // ---- prologue
   load_a(0);
@@ -269,6 +279,13 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       const int r16 = (lane >> 5) + 2 * i;
       const int crow = s_crow[mb * 16 + r16];
       f32x4 v = *(const f32x4*)(slab + r16 * RED_RS + fpos);
+      if (p.splits > 1) {
+        // K is split: the fp32 partial tile [row 64][column 512] goes to scratch with plain stores; the reduction
+        // kernel launched behind this one adds the splits and finishes the rows
+        if (fcol_ok && crow >= 0)
+          *(f32x4*)(p.ctmp + (((int64_t)tile * p.splits + split) * MD_BM + mb * 16 + r16) * 512 + wv * 128 + fc4) = v;
+        continue;
+      }
       if (fcol_ok && crow >= 0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
@@ -289,6 +306,73 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   }
 }
 
+// Second pass of a split-K launch of mid_kernel: out tile = sum over splits of the fp32 partial tiles (in split order,
+// so the result does not depend on timing), then channel scale, bias, routing weight, conversion and the row scatter
+// exactly as mid_kernel's own epilogue does.  One workgroup per (tile, 16-row block); thread -> 4 columns of 2 rows per pass.
+template <int DT, bool CHANNEL, bool MOE>
+__global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
+  const int t = threadIdx.x;
+  const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
+  const int tile = blockIdx.x >> 2, rb = blockIdx.x & 3;
+  const int mt = tile % mtiles, nt4 = tile / mtiles;
+  const int row0 = mt * MD_BM;
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  if (MOE) {
+    if (row0 >= *p.ntpp) return;
+    const int e = p.expert_ids[mt];
+    if (e < 0) return;
+    Sc += e * p.s_estride;
+    if (bias) bias += e * p.n_estride;
+  }
+  const int fc4 = (t & 127) * 4;
+  const int ncol = nt4 * 512 + fc4;
+  if (ncol >= p.N) return;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  {
+    const int base = ncol & ~31, cl = ncol & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  }
+  const float* parts = p.ctmp + (int64_t)tile * p.splits * (MD_BM * 512) + fc4;
+#pragma unroll 2
+  for (int i = 0; i < 8; ++i) {
+    const int r = rb * 16 + (t >> 7) + 2 * i;
+    int crow = -1;
+    if (MOE) {
+      const int id = p.sorted_ids[row0 + r];
+      if ((unsigned)id < (unsigned)p.c_rows) crow = id;
+    } else if (row0 + r < p.M) {
+      crow = row0 + r;
+    }
+    if (crow < 0) continue;
+    f32x4 v = {0, 0, 0, 0};
+    for (int sidx = 0; sidx < p.splits; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+    if (MOE && p.mul_topk) {
+      const float tw = p.topk_w[crow];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] *= tw;
+    }
+    u32x2 o;
+    if constexpr (DT == DT_F16)
+      o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+    else
+      o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+    *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+  }
+}
+
 typedef void (*mid_fn)(const KParams);
 
 template <int DT, bool MOE>
@@ -296,20 +380,31 @@ static mid_fn pick_mid2(bool zp, bool channel) {
   if (zp) return channel ? mid_kernel<DT, true, true, MOE> : mid_kernel<DT, true, false, MOE>;
   return channel ? mid_kernel<DT, false, true, MOE> : mid_kernel<DT, false, false, MOE>;
 }
+template <int DT, bool MOE>
+static mid_fn pick_reduce(bool channel) {
+  return channel ? mid_reduce_kernel<DT, true, MOE> : mid_reduce_kernel<DT, false, MOE>;
+}
 
 int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
-  mid_fn fn;
-  if (a->dtype == DT_F16)
+  mid_fn fn, red;
+  if (a->dtype == DT_F16) {
     fn = moe ? pick_mid2<DT_F16, true>(zp, channel) : pick_mid2<DT_F16, false>(zp, channel);
-  else
+    red = moe ? pick_reduce<DT_F16, true>(channel) : pick_reduce<DT_F16, false>(channel);
+  } else {
     fn = moe ? pick_mid2<DT_BF16, true>(zp, channel) : pick_mid2<DT_BF16, false>(zp, channel);
+    red = moe ? pick_reduce<DT_BF16, true>(channel) : pick_reduce<DT_BF16, false>(channel);
+  }
   KParams p = make_kparams(a, pl);
-  const int64_t grid = (int64_t)pl.tiles;
+  const int64_t grid = (int64_t)pl.tiles * pl.splits;
   if (grid <= 0) return 0;
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), MD_SMEM, stream, p);
   W4A16_HIP(hipGetLastError());
+  if (pl.splits > 1) {
+    hipLaunchKernelGGL(red, dim3((unsigned)(pl.tiles * 4)), dim3(256), 0, stream, p);
+    W4A16_HIP(hipGetLastError());
+  }
   return 0;
 }
 
