@@ -223,3 +223,24 @@ def test_prefill_llama_o_proj_bf16_awq(ops, dev, workspace):
     a = _a(size_m, size_k, torch.bfloat16, dev, seed=42)
     out = run_gemm(ops, layer, a, dev, workspace)
     check_close(out, a, layer)
+
+
+@pytest.mark.parametrize("dtype,mode", [(torch.float16, "gptq"), (torch.bfloat16, "awq")])
+def test_mid_kernel_split_k(ops, dev, workspace, dtype, mode):
+    """1024 x 4096 output = 128 tiles of 64 x 512: the 64-row kernel runs with K split in two and the reduction pass."""
+    size_m, size_k, size_n = 1024, 2048, 4096
+    layer = make_layer(size_k, size_n, 128, dtype, has_zp=(mode == "awq"), seed=21, rule="absmax7" if mode == "gptq" else "minmax")
+    a = _a(size_m, size_k, dtype, dev)
+    bias = torch.randn(size_n, generator=torch.Generator().manual_seed(3)).to(dtype)
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias.to(dev)))
+    check_close(out, a, layer, bias=bias)
+    out2 = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias.to(dev)))
+    assert torch.equal(out, out2)
+    # one-hot rows stay exact through the split (one split holds the product, the others add zero)
+    ks = torch.randperm(size_k, generator=torch.Generator().manual_seed(1))[:size_m // 2]
+    oh = torch.zeros(size_m, size_k, dtype=dtype)
+    oh[torch.arange(size_m // 2), ks] = 1.0
+    out = run_gemm(ops, layer, oh.to(dev), dev, workspace)
+    assert torch.equal(out[:size_m // 2].cpu(), layer.w_ref[ks])
+    assert int(out[size_m // 2:].abs().sum()) == 0

@@ -147,6 +147,33 @@ def test_moe_gemm_equals_oracle(dev, m, topk, e, bs, variant, mul):
     assert int(ws.abs().sum()) == 0
 
 
+def test_moe_gemm_split_k_blocks_of_64(dev):
+    """Enough rows for blocks of 64 but fewer than 256 tiles: the 64-row kernel splits K and runs its reduction pass."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    m, topk, e, bs, k, n = 2048, 2, 4, 64, 2048, 1024
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, 128, torch.float16, False, False, seed=50)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).half()
+    ids = rand_topk(m, topk, e, seed=6)
+    tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7))
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e)
+    ws = marlin_make_workspace_new(dev, 4)
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), None, mq.to(dev), None, ms.to(dev), None, mz.to(dev), gi.to(dev), perm.to(dev), ws, s, x, t,
+        tw.to(dev), moe_block_size=bs, top_k=topk, mul_topk_weights=True, is_ep=False, b_q_type=scalar_types.uint4b8,
+        size_m=m, size_n=n, size_k=k, is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
+    # dense reference per expert on the gathered rows
+    flat = ids.flatten().long()
+    ref = torch.zeros(m * topk, n)
+    for ex in range(e):
+        rows = torch.nonzero(flat == ex).flatten()
+        ref[rows] = (a[rows // topk].float() @ layers[ex].w_ref.float()) * tw.flatten()[rows].unsqueeze(1)
+    mtr = gr.error_metrics(out, ref)
+    assert mtr["max_rel"] <= 2e-2 and mtr["mean_rel"] < 0.04, mtr
+
+
 def test_moe_gemm_skips_foreign_experts_and_bias(dev):
     """expert_ids = -1 blocks are left untouched (expert parallelism); per-expert bias is added."""
     import vllm_amd.ops as ops
