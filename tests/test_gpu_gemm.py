@@ -244,3 +244,21 @@ def test_mid_kernel_split_k(ops, dev, workspace, dtype, mode):
     out = run_gemm(ops, layer, oh.to(dev), dev, workspace)
     assert torch.equal(out[:size_m // 2].cpu(), layer.w_ref[ks])
     assert int(out[size_m // 2:].abs().sum()) == 0
+
+
+def test_reduce_flags_do_not_change_results(ops, dev, workspace):
+    """use_atomic_add / use_fp32_reduce are accepted for interface parity (test_marlin_gemm.py:62-63); partial sums are
+    always fp32 and added in a fixed order, so every combination gives the same bits."""
+    import vllm_amd.scalar_type as vst
+    layer = make_layer(4096, 512, 128, torch.float16, seed=31, rule="absmax7", w_std=0.05)
+    a = _a(16, 4096, torch.float16, dev)
+    outs = []
+    for atomic in (False, True):
+        for fp32 in (False, True):
+            outs.append(ops.gptq_marlin_gemm(a, None, layer.marlin_q.to(dev), None, layer.marlin_s.to(dev), None,
+                                             layer.marlin_zp.to(dev), layer.g_idx_sorted.to(dev), layer.sort_indices.to(dev),
+                                             workspace, vst.scalar_types.uint4b8, 16, 512, 4096, is_k_full=True,
+                                             use_atomic_add=atomic, use_fp32_reduce=fp32, is_zp_float=False))
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    check_close(outs[0], a, layer)
