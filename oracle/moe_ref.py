@@ -67,6 +67,27 @@ def topk_softmax(gating_output: torch.Tensor, topk: int, renormalize: bool):
     return w, ids, src
 
 
+def batched_moe_align_block_size(max_tokens_per_batch: int, block_size: int, expert_num_tokens: torch.Tensor):
+    """Alignment for per-expert batches, as the reference's test states it
+    (tests/kernels/moe/test_moe_align_block_size.py:316-352) and its docstring example
+    (moe_align_block_size.py:117-149): rows e*MAX + j for j < n_e, experts padded to block_size with the value
+    E*MAX, empty experts skipped, expert_ids -1 past the end."""
+    e = expert_num_tokens.numel()
+    padded = -(-max_tokens_per_batch // block_size) * block_size * e
+    sentinel = e * max_tokens_per_batch
+    sorted_ids = torch.full((padded,), sentinel, dtype=torch.int32)
+    expert_ids = torch.full((padded // block_size,), -1, dtype=torch.int32)
+    i = 0
+    for ex, nt in enumerate(expert_num_tokens.tolist()):
+        first = i
+        for j in range(nt):
+            sorted_ids[i] = ex * max_tokens_per_batch + j
+            i += 1
+        i = -(-i // block_size) * block_size
+        expert_ids[first // block_size:i // block_size] = ex
+    return sorted_ids, expert_ids, torch.tensor([i], dtype=torch.int32)
+
+
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
     d = x.shape[-1] // 2
     return torch.nn.functional.silu(x[..., :d]) * x[..., d:]

@@ -109,6 +109,21 @@ def test_topk_softmax_ties_take_lowest_index(dev):
     assert torch.allclose(w[0].cpu(), torch.full((3,), 1 / 3))
 
 
+@pytest.mark.parametrize("max_tokens", [13, 64, 512])
+@pytest.mark.parametrize("e", [8, 32])
+@pytest.mark.parametrize("bs", [8, 16, 64])
+@pytest.mark.parametrize("empty", [False, True])
+def test_batched_align_equals_oracle(dev, max_tokens, e, bs, empty):
+    from vllm_amd.moe_align_block_size import batched_moe_align_block_size
+    g = torch.Generator().manual_seed(max_tokens + e)
+    n = torch.randint(1, max_tokens + 1, (e,), generator=g, dtype=torch.int32)
+    if empty:
+        n[torch.randperm(e, generator=g)[:e // 2]] = 0
+    s, x, t = batched_moe_align_block_size(max_tokens, bs, n.to(dev))
+    ws, wx, wt = mr.batched_moe_align_block_size(max_tokens, bs, n)
+    assert torch.equal(t.cpu(), wt) and torch.equal(s.cpu(), ws) and torch.equal(x.cpu(), wx)
+
+
 # ------------------------------------------------------------------------------------- MoE GEMM
 def make_experts(e, k, n, group, dtype, has_zp, act_order, seed):
     layers = [make_layer(k, n, group, dtype, has_zp=has_zp, act_order=act_order, seed=seed + i, w_std=0.1) for i in range(e)]
@@ -263,3 +278,33 @@ def test_fused_marlin_moe_mixtral_shape(dev):
             act = (torch.nn.functional.silu(h[:inter].float()).to(dtype) * h[inter:])
             ref[t] += float(tw[t, j]) * (act.float() @ w2[ex]).to(dtype).float()
     torch.testing.assert_close(out.cpu().float(), ref, atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_batched_fused_marlin_moe_equals_standard(dev, dtype):
+    """The reference's own check (tests/kernels/moe/test_moe.py:977-1135): batching tokens per expert and running the
+    batched entry point gives what fused_marlin_moe gives for the same tokens (atol 1e-3)."""
+    from vllm_amd.fused_marlin_moe import batched_fused_marlin_moe, fused_marlin_moe
+    e, k, inter, max_tokens = 4, 256, 128, 70
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=500)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 128, dtype, False, False, seed=600)
+    g = torch.Generator().manual_seed(13)
+    n = torch.tensor([70, 0, 33, 64], dtype=torch.int32)
+    x = (torch.randn(e, max_tokens, k, generator=g) / 10).to(dtype)
+    out = batched_fused_marlin_moe(x.to(dev), n.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), None,
+                                   quant_type_id=l1[0].type_id)
+    assert out.shape == (e, max_tokens, k)
+    # the same tokens through the standard entry point: token i of expert ex routed to ex with weight 1
+    for ex in range(e):
+        cnt = int(n[ex])
+        if cnt == 0:
+            continue
+        tok = x[ex, :cnt].contiguous().to(dev)
+        ids = torch.full((cnt, 1), ex, dtype=torch.int32, device=dev)
+        ones = torch.ones(cnt, 1, dtype=torch.float32, device=dev)
+        want = fused_marlin_moe(tok, q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), None, ones, ids,
+                                quant_type_id=l1[0].type_id, global_num_experts=e)
+        torch.testing.assert_close(out[ex, :cnt], want, atol=1e-3, rtol=0)
+        ref = mr.torch_experts(x[ex, :cnt], torch.stack([l.w_ref.t() for l in l1]), torch.stack([l.w_ref.t() for l in l2]),
+                               torch.ones(cnt, 1), torch.full((cnt, 1), ex))
+        torch.testing.assert_close(out[ex, :cnt].cpu().float(), ref.float(), atol=5e-2, rtol=0)

@@ -110,3 +110,12 @@ def test_topk_softmax_hand_case_and_torch_agreement():
     tw, ti = torch.topk(torch.softmax(x, -1), 4)
     assert torch.equal(ids.long(), ti) and torch.allclose(w, tw / tw.sum(-1, keepdim=True), atol=1e-6)
     assert src.tolist() == [[k * 9 + r for k in range(4)] for r in range(9)]
+
+
+def test_batched_align_docstring_example():
+    """Worked example of the reference's docstring (moe_align_block_size.py:117-149)."""
+    s, x, t = mr.batched_moe_align_block_size(8, 4, torch.tensor([2, 3, 0, 6, 8]))
+    assert s[:28].tolist() == [0, 1, 40, 40, 8, 9, 10, 40, 24, 25, 26, 27, 28, 29, 40, 40, 32, 33, 34, 35, 36, 37, 38, 39,
+                               40, 40, 40, 40]
+    assert x.tolist() == [0, 1, 3, 3, 4, 4, -1, -1, -1, -1]
+    assert int(t) == 24 and s.numel() == 40

@@ -7,7 +7,7 @@ import torch
 
 from . import _custom_ops as ops
 from .marlin_utils import marlin_make_workspace_new
-from .moe_align_block_size import moe_align_block_size
+from .moe_align_block_size import batched_moe_align_block_size, moe_align_block_size
 from .scalar_type import ScalarType, scalar_types
 
 
@@ -122,3 +122,53 @@ def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, ga
         ops.moe_sum(moe_output.contiguous(), output)
         return output
     return moe_sum(moe_output, output)
+
+
+def batched_fused_marlin_moe(hidden_states, expert_num_tokens, w1, w2, bias1, bias2, w1_scale, w2_scale, gating_output,
+                             quant_type_id: int, apply_router_weight_on_input: bool = False,
+                             global_num_experts: int = -1, activation: str | None = "silu", expert_map=None,
+                             global_scale1=None, global_scale2=None, g_idx1=None, g_idx2=None, sort_indices1=None,
+                             sort_indices2=None, w1_zeros=None, w2_zeros=None, workspace=None,
+                             intermediate_cache13=None, intermediate_cache2=None, is_k_full: bool = True, output=None,
+                             inplace: bool = False) -> torch.Tensor:
+    """MoE over activations already batched per expert, hidden_states [E, max_tokens, K] with expert_num_tokens[e]
+    valid rows in batch e (reference fused_marlin_moe.py:343-498): the batch is viewed as [E * max_tokens, K] with
+    top_k = 1 and unit routing weights, and the alignment comes from the row counts.  Returns [E, max_tokens, K];
+    rows past expert_num_tokens[e] are not written."""
+    assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K]. But got {hidden_states.size()}"
+    if inplace:
+        assert output is None, "Conflicting request."
+    quant_type = ScalarType.from_id(quant_type_id)
+    assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128), \
+        f"unsupported MoE weight type {quant_type}"
+    num_bits = quant_type.size_bits
+    B, batch_tokens_max, K = hidden_states.size()
+    M = B * batch_tokens_max
+    E = w1.size(0)
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    assert expert_num_tokens.size(0) == E
+    assert B == E, "Batch must be as big as number of experts as the tokens are sorted into the batch/expert they belong to"
+    assert w1.size(1) * 16 == K, "Hidden size mismatch w1"
+    assert w2.size(2) // (num_bits // 2) == K, "Hidden size mismatch w2"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert activation is not None
+    topk = 1
+    block_size_m = 64
+    sorted_token_ids, expert_ids, num_tokens_post_padded = batched_moe_align_block_size(
+        max_tokens_per_batch=batch_tokens_max, block_size=block_size_m, expert_num_tokens=expert_num_tokens)
+    if output is None and inplace:
+        output = hidden_states
+    topk_weights = torch.ones((M, topk), device=hidden_states.device, dtype=torch.float32)
+    output = _fused_marlin_moe(
+        hidden_states=hidden_states.view(-1, K), w1=w1, w2=w2, bias1=bias1, bias2=bias2, w1_scale=w1_scale,
+        w2_scale=w2_scale, topk_weights=topk_weights, num_topk=topk, quant_type=quant_type,
+        apply_router_weight_on_input=apply_router_weight_on_input, activation=activation, expert_map=expert_map,
+        block_size_m=block_size_m, sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
+        num_tokens_post_padded=num_tokens_post_padded, global_scale1=global_scale1, global_scale2=global_scale2,
+        g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2, w1_zeros=w1_zeros,
+        w2_zeros=w2_zeros, workspace=workspace, intermediate_cache13=intermediate_cache13,
+        intermediate_cache2=intermediate_cache2, output=output.view(-1, K) if output is not None else output,
+        is_k_full=is_k_full)
+    return output.view(B, batch_tokens_max, K)
