@@ -308,3 +308,30 @@ def test_batched_fused_marlin_moe_equals_standard(dev, dtype):
         ref = mr.torch_experts(x[ex, :cnt], torch.stack([l.w_ref.t() for l in l1]), torch.stack([l.w_ref.t() for l in l2]),
                                torch.ones(cnt, 1), torch.full((cnt, 1), ex))
         torch.testing.assert_close(out[ex, :cnt].cpu().float(), ref.float(), atol=5e-2, rtol=0)
+
+
+def test_fused_marlin_moe_with_bias(dev):
+    """Per-expert biases on both GEMMs (reference tests/kernels/moe/test_moe.py:750-830), atol 5e-2."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    dtype, e, topk, m, k, inter = torch.float16, 4, 2, 37, 256, 128
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=700)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 128, dtype, False, False, seed=800)
+    g = torch.Generator().manual_seed(14)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    b1 = (torch.randn(e, 2 * inter, generator=g) / 10).to(dtype)
+    b2 = (torch.randn(e, k, generator=g) / 10).to(dtype)
+    score = torch.randn(m, e, generator=g)
+    tw, ti = torch.topk(torch.softmax(score, dim=-1), topk)
+    pb1 = torch.stack([marlin_permute_bias(b1[i].to(dev)) for i in range(e)])
+    pb2 = torch.stack([marlin_permute_bias(b2[i].to(dev)) for i in range(e)])
+    out = fused_marlin_moe(a.to(dev), q1.to(dev), q2.to(dev), pb1, pb2, s1.to(dev), s2.to(dev), score.to(dev), tw.to(dev),
+                           ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e)
+    ref = torch.zeros(m, k)
+    for t in range(m):
+        for j in range(topk):
+            ex = int(ti[t, j])
+            h = (a[t].float() @ l1[ex].w_ref.float() + b1[ex].float()).to(dtype)
+            act = torch.nn.functional.silu(h[:inter].float()).to(dtype) * h[inter:]
+            ref[t] += float(tw[t, j]) * (act.float() @ l2[ex].w_ref.float() + b2[ex].float()).to(dtype).float()
+    torch.testing.assert_close(out.cpu().float(), ref, atol=5e-2, rtol=0)
