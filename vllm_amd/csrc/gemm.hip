@@ -73,6 +73,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
 
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   const bool w8 = a->wtype == W4A16_WTYPE_U8B128;  // 8-bit weights: general kernel only
+  const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (w8 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
   if (moe) {
@@ -101,7 +102,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
-  if (!moe && !w8 && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  if (!moe && !w8 && pow2_group && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
@@ -138,7 +139,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     int kps = (int)ceil_div(pl.total_ksteps, sp);
     kps = (kps + 3) / 4 * 4;
     sp = (int)ceil_div(pl.total_ksteps, kps);
-    const bool mid_shape = !w8 && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+    const bool mid_shape = !w8 && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
                            (moe ? a->moe_block_size == 64
                                 : (a->size_m > 32 && mid_tiles >= cus / 2));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {

@@ -20,6 +20,7 @@ struct KParams {
   int c_rows;  // rows of C (M, or M*top_k for MoE)
   int N, K;
   int group_ksteps;  // GM_GROUPED: group_size / 32
+  int group_shift;   // log2(group_ksteps) when that is a power of two, else -1
   int ncp;           // column pairs = ceil(N / 128)
   int splits, ksteps_per_split, total_ksteps;
   int xcd_map;
@@ -84,6 +85,9 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.N = (int)a->size_n;
   p.K = (int)a->size_k;
   p.group_ksteps = pl.group_ksteps;
+  p.group_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == pl.group_ksteps) p.group_shift = sh;
   p.ncp = pl.ncp;
   p.splits = pl.splits;
   p.ksteps_per_split = pl.kps;

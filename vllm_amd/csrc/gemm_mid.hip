@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   auto issue = [&](Stage& s, int ks) {  // ks: relative to ks_b
     ks = min(ks_b + ks, ks_e - 1);
     int gi = 0;
-    if (!CHANNEL) gi = ks / p.group_ksteps;
+    if (!CHANNEL) gi = ks >> p.group_shift;  // the host only picks this kernel for power-of-two group sizes
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
