@@ -391,7 +391,10 @@ def main():
     avg_launch_s = sec_per_step / 4
 
     result = {
-        "metric": "W4A16 GEMM algorithmic HBM GB/s, Llama-3-8B decode linears (qkv,o,gate_up,down)",
+        "metric": "W4A16 GEMM \u00b5s + %HBM roofline (M\u226416), %MFMA peak (M=4096), Llama-3-8B shapes",
+        "metric_detail": "value = algorithmic HBM bytes per second over one decode step = the four Llama-3-8B linears "
+                         "(qkv, o, gate_up, down) at M=16; per-shape microseconds and roofline fractions are in "
+                         "`detail` and `summary`",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": timed_steps, "warmup": args.warmup,
         "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
@@ -431,6 +434,12 @@ def main():
         torch.cuda.empty_cache()
         detail["repack"] = bench_repack(ops, dev)
         result["detail"] = detail
+        result["summary"] = {
+            "decode_fp16_gptq_us": {k: round(v["us"], 2) for k, v in detail["decode_fp16_gptq"].items()},
+            "decode_fp16_gptq_hbm_frac": {k: round(v["hbm_frac"], 3) for k, v in detail["decode_fp16_gptq"].items()},
+            "prefill_bf16_awq_us": {k: round(v["us"], 1) for k, v in detail["prefill_bf16_awq"].items()},
+            "prefill_bf16_awq_mfma_frac": {k: round(v["mfma_frac"], 3) for k, v in detail["prefill_bf16_awq"].items()},
+        }
         if args.table:
             with open(args.table, "w") as f:
                 json.dump(detail, f, indent=1)
