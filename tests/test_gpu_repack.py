@@ -84,3 +84,22 @@ def test_repack_errors(ops, dev):
         ops.gptq_marlin_repack(q, e, 256, 64, 4)        # shape mismatch
     with pytest.raises(RuntimeError):
         ops.awq_marlin_repack(q, 128, 64, 3)            # bad bits
+
+
+@pytest.mark.parametrize("num_bits", [4, 8])
+def test_moe_repack_wrappers(ops, dev, num_bits):
+    """Per-expert repack loops (reference vllm/_custom_ops.py:1221-1260): [E, K/pf, N] -> [E, K/16, N * bits / 2]."""
+    e, size_k, size_n = 3, 128, 192
+    g = torch.Generator().manual_seed(17)
+    q = torch.randint(0, 1 << num_bits, (e, size_k, size_n), generator=g, dtype=torch.int32)
+    perm = torch.stack([torch.randperm(size_k, generator=g) for _ in range(e)]).to(torch.int32)
+    layout = ml.marlin_weights_closed_form if num_bits == 4 else ml.marlin_weights_closed_form8
+    packed = torch.stack([qu.pack_rows(q[i], num_bits) for i in range(e)])
+    got = ops.gptq_marlin_moe_repack(packed.to(dev), perm.to(dev), size_k, size_n, num_bits)
+    assert tuple(got.shape) == (e, size_k // 16, size_n * num_bits // 2)
+    for i in range(e):
+        assert torch.equal(got[i].cpu(), layout(q[i], perm[i]))
+    packed = torch.stack([qu.awq_pack(q[i], num_bits) for i in range(e)])
+    got = ops.awq_marlin_moe_repack(packed.to(dev), perm.to(dev), size_k, size_n, num_bits)
+    for i in range(e):
+        assert torch.equal(got[i].cpu(), layout(q[i]))
