@@ -117,6 +117,14 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = pl.total_ksteps;
     pl.xcd_map = 0;
     pl.ctmp_bytes = 0;
+    // One workgroup fills a compute unit, so tiles run in rounds of `cus`.  When the last round is at most half full
+    // and consists of whole 512-column strips (tiles are ordered M first), those strips go to the 64-row kernel instead:
+    // twice as many, half-size workgroups occupy every compute unit for about two thirds of a round.
+    {
+      const int64_t rounds = tiles / cus, tail = tiles - rounds * cus;
+      if (rounds >= 1 && tail > 0 && tail * 2 <= cus && tail % pl.mtiles == 0 && forced_kind != 2)
+        pl.tail_strips = (int)(tail / pl.mtiles);
+    }
     return 0;
   }
 
@@ -266,7 +274,21 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
     b.lda = args->size_k;
     pl.use_perm = false;
   }
-  if (pl.kind == 2) return launch_fat(&b, pl, (hipStream_t)stream);
+  if (pl.kind == 2) {
+    if (pl.tail_strips == 0) return launch_fat(&b, pl, (hipStream_t)stream);
+    Plan head = pl, tail = pl;
+    head.ncp = pl.ncp - pl.tail_strips;
+    head.tiles = head.ncp * pl.mtiles;
+    if (int rc = launch_fat(&b, head, (hipStream_t)stream)) return rc;
+    tail.kind = 3;
+    tail.mb = 4;
+    tail.bm = 64;
+    tail.mtiles = (int)ceil_div(args->size_m, 64);
+    tail.ncp = pl.tail_strips;
+    tail.tiles = tail.mtiles * tail.ncp;
+    tail.strip0 = head.ncp;
+    return launch_mid(&b, tail, (hipStream_t)stream);
+  }
   if (pl.kind == 3) return launch_mid(&b, pl, (hipStream_t)stream);
   return pl.kind == 1 ? launch_decode(&b, pl, (hipStream_t)stream) : launch_skinny(&b, pl, (hipStream_t)stream);
 }

@@ -25,6 +25,7 @@ struct KParams {
   int splits, ksteps_per_split, total_ksteps;
   int xcd_map;
   int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
+  int strip0;    // 64-row kernel: first 512-column strip of this launch (it may finish what the prefill kernel left)
   // MoE
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
@@ -94,6 +95,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.total_ksteps = pl.total_ksteps;
   p.xcd_map = pl.xcd_map;
   p.tn = pl.tn;
+  p.strip0 = pl.strip0;
   p.sorted_ids = a->sorted_token_ids;
   p.expert_ids = a->expert_ids;
   p.ntpp = a->num_tokens_past_padded;

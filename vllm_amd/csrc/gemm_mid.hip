@@ -46,8 +46,9 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   // (MoE: neighbouring blocks mostly belong to the same expert)
   const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
   const int mt = blockIdx.x % mtiles;
-  const int split = (blockIdx.x / mtiles) % p.splits, nt4 = blockIdx.x / (mtiles * p.splits);
-  const int tile = nt4 * mtiles + mt;          // index of the output tile (partials)
+  const int split = (blockIdx.x / mtiles) % p.splits, st_l = blockIdx.x / (mtiles * p.splits);
+  const int tile = st_l * mtiles + mt;         // index of the output tile inside this launch (partials)
+  const int nt4 = p.strip0 + st_l;             // 512-column strip
   const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
   const int row0 = mt * MD_BM;
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   const int t = threadIdx.x;
   const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
   const int tile = blockIdx.x >> 2, rb = blockIdx.x & 3;
-  const int mt = tile % mtiles, nt4 = tile / mtiles;
+  const int mt = tile % mtiles, nt4 = p.strip0 + tile / mtiles;
   const int row0 = mt * MD_BM;
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint16_t* bias = (const uint16_t*)p.bias;

@@ -14,6 +14,8 @@ struct Plan {
   int xcd_map;
   int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel, 3: 64-row ("mid") kernel
   int tn;    // tile width in columns (128; the decode kernel also has 64)
+  int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
+  int tail_strips = 0; // prefill plan: trailing 512-column strips handed to the 64-row kernel (0 = none)
   int64_t ctmp_bytes;  // fp32 split-K partials
   int64_t atmp_bytes;  // column-permuted copy of A (act-order in front of the prefill kernel), after the partials
 };
