@@ -108,9 +108,10 @@ def gemm(ops, wtype, a, layer, workspace):
                                 a.shape[0], layer["n"], layer["k"], True, False, True, False)
 
 
-def time_graph(fn_list, reps, warmup):
+def time_graph(fn_list, reps, warmup, stats=False):
     """Capture `fn_list` (a list of zero-arg launch closures) into one HIP graph, replay it `warmup`
-    times untimed and `reps` times between two events on the launch stream; returns seconds/replay."""
+    times untimed and `reps` times, every replay between its own pair of events on the launch stream;
+    returns the median seconds/replay (with stats=True: (median, min))."""
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
@@ -124,13 +125,15 @@ def time_graph(fn_list, reps, warmup):
         for _ in range(warmup):
             graph.replay()
         torch.cuda.synchronize()
-        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0.record(stream)
-        for _ in range(reps):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        evs[0].record(stream)
+        for i in range(reps):
             graph.replay()
-        t1.record(stream)
+            evs[i + 1].record(stream)
         torch.cuda.synchronize()
-    return t0.elapsed_time(t1) * 1e-3 / reps
+    ts = sorted(evs[i].elapsed_time(evs[i + 1]) * 1e-3 for i in range(reps))
+    med = ts[len(ts) // 2] if len(ts) % 2 else 0.5 * (ts[len(ts) // 2 - 1] + ts[len(ts) // 2])
+    return (med, ts[0]) if stats else med
 
 
 def copies_needed(weight_bytes):
@@ -148,15 +151,18 @@ def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=4
     out = gemm(ops, wtype, a, base, workspace)
     ref = a.float() @ base["w_deq"].float()
     err = float((out.float() - ref).abs().max() / ref.abs().max())
+    mean_rel = float((out.float() - ref).abs().mean() / ref.abs().mean())
     fns = [(lambda c=copies[i % ncopy]: gemm(ops, wtype, a, c, workspace)) for i in range(max(launches, ncopy))]
-    sec = time_graph(fns, reps=3, warmup=1) / len(fns)
-    warm = time_graph([lambda: gemm(ops, wtype, a, base, workspace)] * 20, reps=3, warmup=1) / 20
+    sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=5, warmup=1, stats=True))
+    warm = time_graph([lambda: gemm(ops, wtype, a, base, workspace)] * 20, reps=5, warmup=1) / 20
     by, fl = algorithmic_bytes(m, k, n, zp=zp), 2.0 * m * n * k
     del copies
     torch.cuda.empty_cache()
-    return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_warm": warm * 1e6, "GBps": by / sec / 1e9,
+    return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_min": sec_min * 1e6, "us_warm": warm * 1e6,
+            "launches_timed": 5 * len(fns), "GBps": by / sec / 1e9,
             "TFLOPs": fl / sec / 1e12, "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS,
-            "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS, "max_rel_err": err}
+            "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS, "max_rel_err": err,
+            "mean_rel_err": mean_rel}
 
 
 def make_gptq_actorder_layer(ops, k, n, dtype, dev, seed):
@@ -269,9 +275,21 @@ def bench_moe(ops, wtype, dev):
     return out
 
 
-def cpu_baseline(m, budget_s=12.0):
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(m, budget_s=12.0, matmul_only_budget_s=4.0):
     """The oracle's CPU path (unpack GPTQ nibbles, (q-8)*s group-broadcast, torch.matmul in fp32) on the
-    host cores: whole passes over the four layers at M=`m`, repeated until `budget_s` seconds of CPU work."""
+    host cores: whole passes over the four layers at M=`m`, repeated until `budget_s` seconds of CPU work
+    (`value`, median pass); then the matmul alone on cached dequantised weights (`matmul_only_*`)."""
     from oracle import gemm_ref as gr
     from oracle import quant_utils as qu
     torch.manual_seed(0)
@@ -280,20 +298,39 @@ def cpu_baseline(m, budget_s=12.0):
         q = torch.randint(0, 16, (k, n), dtype=torch.int32)
         layers[name] = (qu.gptq_pack(q), (torch.rand(k // GROUP, n) * 0.01 + 0.005).half(), torch.randn(m, k).half())
         del q
-    passes, t_total, b_total = 0, 0.0, 0
-    while t_total < budget_s:
+    step_bytes = sum(algorithmic_bytes(m, k, n) for k, n in LAYERS.values())
+    pass_s, t_total = [], 0.0
+    while t_total < budget_s or len(pass_s) < 3:
+        t_pass = 0.0
         for name, (packed, s, a) in layers.items():
             t0 = time.perf_counter()
             w = gr.dequant_checkpoint(packed, s, None, None, "gptq", torch.float16)
             out = gr.gemm_ref(a, w)
-            t_total += time.perf_counter() - t0
+            t_pass += time.perf_counter() - t0
             del w, out
-            b_total += algorithmic_bytes(m, *LAYERS[name])
-        passes += 1
-    return {"value": b_total / t_total / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{passes} passes of dequantize (unpack, (q-8)*s) + fp32 matmul over the four layers at M={m}, "
-                      f"{t_total:.1f} s of CPU time", "ms_per_step": t_total / passes * 1e3,
-            "host_cpus": os.cpu_count()}
+        pass_s.append(t_pass)
+        t_total += t_pass
+    med = sorted(pass_s)[len(pass_s) // 2]
+    # matmul only: the largest layer's dequantised fp32 weights are 470 MB, so one layer at a time
+    mm_s = {}
+    for name, (packed, s, a) in layers.items():
+        w = gr.dequant_checkpoint(packed, s, None, None, "gptq", torch.float16).float()
+        af, reps, t_mm = a.float(), 0, 0.0
+        torch.matmul(af, w)
+        while t_mm < matmul_only_budget_s / 4 or reps < 3:
+            t0 = time.perf_counter()
+            torch.matmul(af, w)
+            t_mm += time.perf_counter() - t0
+            reps += 1
+        mm_s[name] = t_mm / reps
+        del w
+    mm_step = sum(mm_s.values())
+    return {"value": step_bytes / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(pass_s)} passes of dequantize (unpack, (q-8)*s) + fp32 matmul over the four layers at "
+                      f"M={m}, {t_total:.1f} s of CPU time, median pass",
+            "ms_per_step": med * 1e3, "ms_per_step_min": min(pass_s) * 1e3,
+            "matmul_only_value": step_bytes / mm_step / 1e9, "matmul_only_ms_per_step": mm_step * 1e3,
+            "host_cpus": os.cpu_count(), "cpu_model": _cpu_model()}
 
 
 def main():
@@ -359,32 +396,38 @@ def main():
         for name in LAYERS:
             gemm(ops, scalar_types.uint4b8, acts[name], s[name], workspace)
 
-    steps_per_graph = nsets
-    fns = [(lambda i=i: step(i)) for i in range(steps_per_graph)]
+    # Exactly `--steps` steps are timed: whole graphs of `nsets` steps (one per weight set) plus, when `--steps` is
+    # not a multiple of nsets, one shorter graph for the remainder.  Warm-up replays the same way.
+    def capture(nsteps, stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(nsteps):
+                step(i)
+        return graph
+
+    def run(nsteps, full, parts):
+        for _ in range(nsteps // nsets):
+            full.replay()
+        if nsteps % nsets:
+            parts[nsteps % nsets].replay()
+
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
-        for f in fns:
-            f()
+        for i in range(nsets):
+            step(i)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            for f in fns:
-                f()
-        done = 0
-        while done < args.warmup:
-            graph.replay()
-            done += steps_per_graph
+        full = capture(nsets, stream)
+        parts = {r: capture(r, stream) for r in {args.steps % nsets, args.warmup % nsets} if r}
+        run(args.warmup, full, parts)
         torch.cuda.synchronize()
-        replays = -(-args.steps // steps_per_graph)
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0.record(stream)
-        for _ in range(replays):
-            graph.replay()
+        run(args.steps, full, parts)
         t1.record(stream)
         torch.cuda.synchronize()
-    timed_steps = replays * steps_per_graph
-    sec_per_step = t0.elapsed_time(t1) * 1e-3 / timed_steps
+    timed_steps = args.steps
+    sec_per_step = t0.elapsed_time(t1) * 1e-3 / max(timed_steps, 1)
     step_bytes = sum(algorithmic_bytes(m, k, n) for k, n in LAYERS.values())
     value = step_bytes / sec_per_step / 1e9
     launches = 4 * timed_steps
