@@ -177,7 +177,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these
   // kernels.  One 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~20 GB/s on a 64-column
   // strip with 16-row tiles (instruction-issue bound), ~12 / ~9 GB/s with 32- / 64-row tiles (dequantisation
-  // per element); the whole chip ~4.7 TB/s; summing K-splits across workgroups adds ~2.2 us of dependent
+  // per element); the whole chip ~4.7 TB/s; summing K-splits across workgroups adds ~1.5 us of dependent
   // device-scope round trips plus the last workgroup's pass over the partial tiles.  Only one such workgroup
   // fits a compute unit, so a grid larger than the number of compute units runs in rounds.  Each split needs
   // >= 1 stage per wavefront and one workspace counter per tile.
@@ -201,6 +201,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       const double bytes = (double)tiles * a->size_k * tn / 2.0;
       const double wg_rate = mb == 1 ? (tn == 64 ? 20e3 : 33e3) : mb == 2 ? 12e3 : 9e3;  // bytes per us
       const double chip_rate = 4.7e6;
+      const double t_xchg = 1.5;
       const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
       const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
       for (int sp = 1; sp <= 16; ++sp) {
@@ -213,7 +214,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
         double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
         if (rate > chip_rate) rate = chip_rate;
         // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
-        const double t_fix = sp > 1 ? 2.2 + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
+        const double t_fix = sp > 1 ? t_xchg + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
         const double t = bytes / rate + t_fix;
         if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, mb, t};
       }

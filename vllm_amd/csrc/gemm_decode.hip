@@ -379,13 +379,9 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     for (int j = 0; j < CPT; j += 2) store_coherent2(my_part + fr * TN + fc + j, v[j], v[j + 1]);
   }
   // ---- cross-workgroup reduction: the last split to arrive sums all partials in split order
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  if (t == 0) {
-    const int old = __hip_atomic_fetch_add(&p.locks[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = (old == p.splits - 1);
-  }
+  if (t == 0) s_last = arrive_last(p.locks + tile * p.lock_stride, p.splits);
   __syncthreads();
   if (!s_last) return;
   if (s_crow[fr] >= 0) {
@@ -403,7 +399,6 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     }
     finalize(v);
   }
-  if (t == 0) __hip_atomic_store(&p.locks[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ------------------------------------------------------------------------------------ host side

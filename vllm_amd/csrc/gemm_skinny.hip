@@ -16,7 +16,7 @@
 //                  wavefront-private LDS slab into the MFMA A operand order (no barrier needed)
 //     scales/zeros one 16-byte / 4-byte load per k-step (cache hits after the first of a group)
 //   The 8 partial tiles are summed through LDS.  Splits are summed by the last workgroup to arrive
-//   at the tile's counter in `workspace`, in split order (deterministic); the counter is reset so
+//   at the tile's counter in `workspace`, in split order (deterministic); arrivals are wrapping increments, so
 //   the workspace is all-zero on exit, as the reference requires (csrc/torch_bindings.cpp:255-267).
 // HBM traffic per launch: every weight byte once (K*N/2), scales (K/g)*N*2, C once; A is re-read
 // once per column pair (from L2), split partials move 2 * splits * M * N * 4 bytes.
@@ -472,13 +472,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 
   // ---- cross-workgroup reduction: the last split to arrive sums all partials in split order.
   // The wait makes every partial of this workgroup complete before its arrival is counted.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  if (t == 0) {
-    const int old = __hip_atomic_fetch_add(&p.locks[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = (old == p.splits - 1);
-  }
+  if (t == 0) s_last = arrive_last(p.locks + tile * p.lock_stride, p.splits);
   __syncthreads();
   if (!s_last) return;
   const float* parts = p.ctmp + (int64_t)tile * p.splits * (BM * 128);
@@ -490,7 +486,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       v += load_coherent(parts + (int64_t)s * (BM * 128) + r * 128 + fc4);
     finalize(r, v);
   }
-  if (t == 0) __hip_atomic_store(&p.locks[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ------------------------------------------------------------------------------------ host side

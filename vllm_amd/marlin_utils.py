@@ -57,10 +57,12 @@ def verify_marlin_supports_shape(output_size_per_partition: int, input_size_per_
 
 
 def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1) -> torch.Tensor:
-    """int32 zeros, one counter per compute unit (x max_blocks_per_sm); marlin_utils.py:237-245.
-    The GEMM keeps the all-zero-on-exit invariant, so one workspace serves any number of calls."""
+    """int32 zeros, four counters per compute unit (x max_blocks_per_sm); the reference's function
+    (marlin_utils.py:237-245) allocates one per SM, which the GEMM also accepts: the extra length only lets it place
+    the counters of neighbouring tiles 16 bytes apart.  The GEMM keeps the all-zero-on-exit invariant, so one
+    workspace serves any number of calls."""
     cus = torch.cuda.get_device_properties(device).multi_processor_count
-    return torch.zeros(cus * max_blocks_per_sm, dtype=torch.int, device=device, requires_grad=False)
+    return torch.zeros(4 * cus * max_blocks_per_sm, dtype=torch.int, device=device, requires_grad=False)
 
 
 def marlin_is_k_full(act_order: bool, is_row_parallel: bool) -> bool:
