@@ -482,8 +482,16 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   for (int r = fr; r < BM; r += 16) {
     if (s_crow[r] < 0) continue;
     f32x4 v = {0, 0, 0, 0};
-    for (int s = 0; s < p.splits; ++s)
-      v += load_coherent(parts + (int64_t)s * (BM * 128) + r * 128 + fc4);
+    // four splits' loads are in flight together; summed in split order
+    for (int s0 = 0; s0 < p.splits; s0 += 4) {
+      f32x4 a[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = load_coherent(parts + (int64_t)min(s0 + i, p.splits - 1) * (BM * 128) + r * 128 + fc4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (s0 + i < p.splits) v += a[i];
+    }
     finalize(r, v);
   }
 }
