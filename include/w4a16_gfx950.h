@@ -73,7 +73,8 @@ typedef struct w4a16_gemm_args {
   void* c;                    /* [size_m(*top_k), size_n] dense                           */
   const uint32_t* b_q_weight; /* [E,] [size_k/16, 2*size_n] Marlin layout                 */
   const void* b_scales;       /* [E,] [num_groups, size_n] Marlin-permuted                */
-  const uint32_t* b_zeros;    /* [E,] [num_groups, size_n/8] Marlin-packed, or NULL       */
+  const uint32_t* b_zeros;    /* [E,] [num_groups, size_n/8] Marlin-packed, or NULL;
+                                 with W4A16_F_ZP_FLOAT: fp16 [num_groups, size_n]        */
   const int32_t* g_idx;       /* [E,] [size_k] sorted group of each Marlin row, or NULL   */
   const int32_t* perm;        /* [E,] [size_k] act-order column gather for a, or NULL     */
   const void* b_bias;         /* [E,] [size_n] Marlin-permuted bias, or NULL              */
@@ -100,7 +101,10 @@ enum {
   W4A16_F_USE_ATOMIC_ADD = 2,   /* accepted; the split-K reduction here is always ordered */
   W4A16_F_USE_FP32_REDUCE = 4,  /* accepted; partial sums are always fp32                 */
   W4A16_F_MUL_TOPK_WEIGHTS = 8, /* MoE: scale each output row by its routing weight       */
-  W4A16_F_MOE = 16
+  W4A16_F_MOE = 16,
+  W4A16_F_ZP_FLOAT = 32         /* b_zeros holds fp16 zero points [num_groups, size_n], Marlin-permuted like the
+                                   scales (HQQ; reference is_zp_float, gptq_marlin.cu:866-880): w = q*s - zp*s.
+                                   fp16, uint4, group size 64, dense op only */
 };
 
 /* Bytes of fp32 scratch (c_tmp) a call with these operands may use (0 = none).

@@ -8,6 +8,7 @@ tensors the op actually receives, so layout decode, scale/zero indexing and act-
 are all part of what is checked:
 
   dequant_marlin(...)   Marlin-layout operands  -> w [K, N] in the activation dtype
+  dequant_marlin_float_zp(...)  the same for fp16 zero points (HQQ)
   dequant_checkpoint()  GPTQ / AWQ checkpoint   -> w [K, N]   (the CPU baseline path:
                         unpack nibbles, (q-8)*s or (q-z)*s group-broadcast)
   gemm_ref(a, w)        fp32 matmul (+ bias), result in fp32
@@ -55,6 +56,37 @@ def dequant_marlin(b_q_weight, b_scales, b_zeros, g_idx, size_k, size_n, bias8: 
     else:
         qz = q - ((8 if num_bits == 4 else 128) if bias8 else 0)
     return qz.to(dtype) * s_full
+
+
+def dequant_marlin_float_zp(b_q_weight, b_scales, b_zeros, size_k, size_n):
+    """HQQ operands (uint4 weights, fp16 scales and fp16 zero points, both [G, N] and Marlin-permuted like scales)
+    -> dense fp16 w[K, N] as the reference kernel forms its B operand: zs = half(zp * s) rounded once, then
+    w = fma(q, s, -zs) rounded once (marlin_template.h:174-181 scale_and_sub, :1235-1240).  Computed in float64,
+    where q * s - zs is exact, and rounded to fp16 once.
+
+    The reference's test compares against (q - zp) * s in fp16 tensor arithmetic with a mean-relative gate of 0.04
+    (tests/kernels/quantization/test_marlin_gemm.py:524-535); `float_zp_test_ref` below is that formula.
+    Pinned by (tests/test_oracle_quant.py): hand-computed words where the two roundings differ from the test
+    formula, zp = 0 reducing to the plain q * s product, and agreement with `float_zp_test_ref` to 2 fp16 ulps of
+    max(|q s|, |zp s|) on random data."""
+    q = marlin_unpack_weights(b_q_weight)
+    assert tuple(q.shape) == (size_k, size_n)
+    assert b_scales.dtype == torch.float16 and b_zeros.dtype == torch.float16
+    s = marlin_unpermute_scales(b_scales, True)
+    z = marlin_unpermute_scales(b_zeros, True)
+    zs = (z * s)                                  # fp16 product, one rounding
+    s_full = _expand_groups(s, size_k).double()
+    zs_full = _expand_groups(zs, size_k).double()
+    return (q.double() * s_full - zs_full).to(torch.float16)
+
+
+def float_zp_test_ref(q, scale, zero, group_size: int):
+    """The reference test's dequantisation for HQQ (test_marlin_gemm.py:524-529): q uint8 [N, K], scale and zero
+    fp16 [N, K/group]; returns w [K, N] = ((q - zero) * scale) evaluated in fp16 tensor arithmetic."""
+    n, k = q.shape
+    b_flat = q.reshape(-1, group_size)
+    dequant = (b_flat.to(torch.float16) - zero.reshape(-1, 1)) * scale.reshape(-1, 1)
+    return dequant.reshape(n, k).transpose(1, 0).contiguous()
 
 
 def dequant_checkpoint(qweight, scales, qzeros, g_idx, fmt: str, dtype):

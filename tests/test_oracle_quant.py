@@ -179,3 +179,69 @@ def test_uint8b128_quantizer_and_dequant(dtype, group):
     wg = w.float().view(k // gs, gs, n)
     want = torch.maximum(wg.amax(1).abs() / 127, wg.amin(1).abs() / 128)
     assert torch.allclose(s.float(), want, rtol=2e-2)
+
+
+# ------------------------------------------------------------------ float zero points (HQQ)
+def _hqq_operands(q, s, z):
+    """q int [K, N], s / z fp16 [G, N] -> Marlin operands (group 64)."""
+    k, n = q.shape
+    mq = ml.gptq_marlin_repack(qu.gptq_pack(q.to(torch.int32)), None, k, n)
+    return mq, ml.marlin_permute_scales(s, k, n, 64), ml.marlin_permute_scales(z, k, n, 64)
+
+
+def test_float_zp_reduces_to_integer_zero_points():
+    """s = 1 and integer zero points: every step is exact, so the result is q - z, which is also what the packed
+    integer zero-point path (pinned above against the quantizer's w_ref) gives."""
+    g = torch.Generator().manual_seed(11)
+    k, n = 128, 64
+    q = torch.randint(0, 16, (k, n), generator=g, dtype=torch.int32)
+    z = torch.randint(0, 16, (k // 64, n), generator=g, dtype=torch.int32)
+    s = torch.ones(k // 64, n, dtype=torch.float16)
+    mq, ms, mz = _hqq_operands(q, s, z.half())
+    w = gr.dequant_marlin_float_zp(mq, ms, mz, k, n)
+    assert torch.equal(w, (q - z.repeat_interleave(64, 0)).half())
+    mz_int = ml.marlin_zero_points(z, k // 64, n)
+    assert torch.equal(w, gr.dequant_marlin(mq, ms, mz_int, None, k, n, False, torch.float16))
+
+
+def test_float_zp_zero_is_plain_scaling_and_pow2_scales_match_the_test_formula():
+    g = torch.Generator().manual_seed(12)
+    k, n = 128, 128
+    q = torch.randint(0, 16, (k, n), generator=g, dtype=torch.int32)
+    s = torch.randn(k // 64, n, generator=g).half()
+    z0 = torch.zeros(k // 64, n, dtype=torch.float16)
+    mq, ms, mz = _hqq_operands(q, s, z0)
+    assert torch.equal(gr.dequant_marlin_float_zp(mq, ms, mz, k, n), q.half() * s.repeat_interleave(64, 0))
+    # power-of-two scales: zp * s is exact, and so is (q - zp) * s whenever q - zp is representable
+    s2 = torch.tensor([0.25, 2.0]).half().view(2, 1).expand(2, n).contiguous()
+    z = (torch.randint(0, 64, (k // 64, n), generator=g).half() / 4)            # multiples of 1/4 below 16
+    mq, ms, mz = _hqq_operands(q, s2, z)
+    ref = gr.float_zp_test_ref(q.t().contiguous().to(torch.uint8), s2.t().contiguous(), z.t().contiguous(), 64)
+    assert torch.equal(gr.dequant_marlin_float_zp(mq, ms, mz, k, n), ref)
+
+
+def test_float_zp_hand_derived_rounding_case():
+    """s = zp = 1 + 2^-10, q = 1:  zp*s = 1 + 2^-9 + 2^-20 rounds to 1 + 2^-9;  q*s - zs = -2^-10 exactly.
+    (The reference test's formula (q - zp) * s gives -2^-10 (1 + 2^-10) instead: the kernel's two roundings differ.)"""
+    k, n = 64, 64
+    q = torch.ones(k, n, dtype=torch.int32)
+    v = torch.full((1, n), 1.0 + 2.0 ** -10, dtype=torch.float16)
+    mq, ms, mz = _hqq_operands(q, v, v)
+    w = gr.dequant_marlin_float_zp(mq, ms, mz, k, n)
+    assert torch.equal(w, torch.full((k, n), -(2.0 ** -10), dtype=torch.float16))
+    ref = gr.float_zp_test_ref(q.t().contiguous().to(torch.uint8), v.t().contiguous(), v.t().contiguous(), 64)
+    assert float(ref[0, 0]) == -(2.0 ** -10) * (1 + 2.0 ** -10)
+
+
+def test_float_zp_close_to_the_reference_test_formula():
+    g = torch.Generator().manual_seed(13)
+    k, n = 256, 128
+    q = torch.randint(0, 10, (k, n), generator=g, dtype=torch.int32)             # as the reference test draws them
+    s = torch.randn(k // 64, n, generator=g).half()
+    z = torch.randn(k // 64, n, generator=g).half()
+    mq, ms, mz = _hqq_operands(q, s, z)
+    w = gr.dequant_marlin_float_zp(mq, ms, mz, k, n).float()
+    ref = gr.float_zp_test_ref(q.t().contiguous().to(torch.uint8), s.t().contiguous(), z.t().contiguous(), 64).float()
+    s_full, z_full = s.float().repeat_interleave(64, 0), z.float().repeat_interleave(64, 0)
+    bound = 2.0 ** -9 * torch.maximum((q.float() * s_full).abs(), (z_full * s_full).abs()) + 1e-7
+    assert ((w - ref).abs() <= bound).all()

@@ -211,7 +211,6 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
     _check(b_scales.dim() == 2 and b_scales.size(1) == size_n,
            f"b_scales dim 1 = {b_scales.size(-1)} is not size_n = {size_n}")
     _check(b_scales.dtype == a.dtype, "scalar type of a and b_scales must match")
-    _check(not is_zp_float, "float zero points (HQQ) are not implemented by the gfx950 W4A16 library")
     _check(_opt(global_scale) is None, "global_scale can only be used for nvfp4 format.")
     _check(workspace.is_cuda and workspace.dtype == torch.int32, "workspace must be an int32 GPU tensor")
     num_groups = b_scales.size(0)
@@ -228,11 +227,18 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
     b_zeros = None
     if b_zeros_or_none is not None and b_zeros_or_none.size(-1) > 0:
         b_zeros = b_zeros_or_none
-        _check(b_zeros.is_cuda and b_zeros.is_contiguous() and b_zeros.dtype == torch.int32,
-               "b_zeros is not a contiguous int32 GPU tensor")
+        _check(b_zeros.is_cuda and b_zeros.is_contiguous(), "b_zeros is not a contiguous GPU tensor")
         _check(b_zeros.dim() == 2, f"b_zeros rank = {b_zeros.dim()} is not 2")
         _check(b_zeros.size(0) == num_groups, f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
-        _check(b_zeros.size(1) == size_n // 8, f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // 8}")
+        if is_zp_float:  # HQQ: fp16 zero points shaped and permuted like the scales (gptq_marlin.cu:866-887)
+            _check(a.dtype == torch.float16, "Computation type must be float16 (half) when using float zero points.")
+            _check(b_zeros.dtype == a.dtype, "b_zeros type is not the type of a")
+            _check(b_zeros.size(1) == size_n, f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
+        else:
+            _check(b_zeros.dtype == torch.int32, "b_zeros type is not kInt")
+            _check(b_zeros.size(1) == size_n // 8,
+                   f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // 8}")
+    _check(not is_zp_float or b_zeros is not None, "is_zp_float = True needs b_zeros")
     wtype = _wtype_code(int(b_q_type), b_zeros is not None)
 
     b_bias = _opt(b_bias_or_none)
@@ -254,6 +260,8 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
         flags |= _lib.F_IS_K_FULL
     if use_atomic_add:
         flags |= _lib.F_USE_ATOMIC_ADD
+    if is_zp_float:
+        flags |= _lib.F_ZP_FLOAT
     args = _lib.GemmArgs()
     _fill_common(args, a, c, b_q_weight, b_bias, b_scales, b_zeros, g_idx, perm, workspace, wtype,
                  size_m, size_n, size_k, num_groups, flags)

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libw4a16_gfx950.so")
 W4A16_OK = 0
 WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128 = 0, 1, 2
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
-F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE = 1, 2, 4, 8, 16
+F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE, F_ZP_FLOAT = 1, 2, 4, 8, 16, 32
 
 c_void_p, c_i64, c_i32, c_u32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32
 

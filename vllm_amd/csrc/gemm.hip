@@ -38,6 +38,19 @@ static int validate(const w4a16_gemm_args* a) {
                 "b_q_type must be uint4b8 or uint8b128 when has_zp = False");
   W4A16_CHECK((a->g_idx == nullptr) == (a->perm == nullptr),
               "g_idx and perm must both be given (act-order) or both be empty");
+  if (a->flags & W4A16_F_ZP_FLOAT) {
+    W4A16_CHECK(has_zp, "float zero points requested but b_zeros is null");
+    W4A16_CHECK(a->dtype == W4A16_DTYPE_F16, "Computation type must be float16 (half) when using float zero points.");
+    if (a->flags & W4A16_F_MOE)
+      return fail(W4A16_ENOTIMPL, "float zero points are not implemented for the MoE op in this build");
+    // the reference instantiates float zero points for group size 64 without act-order only
+    // (csrc/quantization/gptq_marlin/gptq_marlin.cu:364-379)
+    W4A16_CHECK(a->g_idx == nullptr && a->num_groups > 0 && a->size_k == a->num_groups * 64,
+                "Unsupported shapes: MNK = [%lld, %lld, %lld], has_act_order = %d, num_groups = %lld, is_zp_float = 1 "
+                "(float zero points need group_size = 64 and no act-order)",
+                (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, a->g_idx != nullptr,
+                (long long)a->num_groups);
+  }
   if (a->flags & W4A16_F_MOE) {
     W4A16_CHECK(a->sorted_token_ids && a->expert_ids && a->num_tokens_past_padded, "null MoE index pointer");
     W4A16_CHECK(a->moe_block_size == 8 || (a->moe_block_size % 16 == 0 && a->moe_block_size >= 16 &&
@@ -72,9 +85,10 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
 
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
-  const bool w8 = a->wtype == W4A16_WTYPE_U8B128;  // 8-bit weights: general kernel only
+  // 8-bit weights and float zero points run on the general (skinny) kernel only
+  const bool general_only = a->wtype == W4A16_WTYPE_U8B128 || (a->flags & W4A16_F_ZP_FLOAT) != 0;
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
-  if (w8 && moe && act_order)
+  if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
   if (moe) {
     const int bs = a->moe_block_size;
@@ -102,7 +116,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
-  if (!moe && !w8 && pow2_group && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  if (!moe && !general_only && pow2_group && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
@@ -147,7 +161,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     int kps = (int)ceil_div(pl.total_ksteps, sp);
     kps = (kps + 3) / 4 * 4;
     sp = (int)ceil_div(pl.total_ksteps, kps);
-    const bool mid_shape = !w8 && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+    const bool mid_shape = !general_only && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
                            (moe ? a->moe_block_size == 64
                                 : (a->size_m > 32 && mid_tiles >= cus / 2));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
@@ -171,7 +185,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
 
   // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
-  const bool decode_shape = !w8 && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
+  const bool decode_shape = !general_only && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
                             (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
 
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these

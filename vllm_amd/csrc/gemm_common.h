@@ -152,6 +152,32 @@ __device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const Col
   }
 }
 
+// Float zero points (HQQ; fp16 only): the B operand is fma(q, s, -zs) with zs = half(zp * s) rounded once, as the
+// reference computes it (marlin_template.h:174-181 scale_and_sub, :1235-1240).  q is made exact first:
+// (1024+q) - 1024 for the low nibbles, (1024+16q)/16 - 64 for the high ones.
+__device__ __forceinline__ void dequant_pair_zpf(uint32_t xa, uint32_t xb, uint32_t s_pair, uint32_t zs_pair,
+                                                 u32x4& o0, u32x4& o1) {
+  const uint32_t MLO = 0x000f000fu, MHI = 0x00f000f0u;
+  uint32_t EX = 0x64006400u;
+  asm("" : "+v"(EX));
+  const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f}, k64 = {(_Float16)64.0f, (_Float16)64.0f};
+  const f16x2 s = as_h2(s_pair), zs = as_h2(zs_pair);
+  const f16x2 s0 = {s.x, s.x}, s1 = {s.y, s.y};
+  const f16x2 nz0 = {-zs.x, -zs.x}, nz1 = {-zs.y, -zs.y};
+  auto lo = [&](uint32_t x, f16x2 sc, f16x2 nz) {
+    const f16x2 q = as_h2((x & MLO) | EX) - k1024;
+    return as_u32(__builtin_elementwise_fma(q, sc, nz));
+  };
+  auto hi = [&](uint32_t x, f16x2 sc, f16x2 nz) {
+    const f16x2 q = as_h2((x & MHI) | EX) * sixteenth - k64;
+    return as_u32(__builtin_elementwise_fma(q, sc, nz));
+  };
+  const uint32_t ya = xa >> 8, yb = xb >> 8;
+  o0 = u32x4{lo(xa, s0, nz0), hi(xa, s0, nz0), lo(xb, s0, nz0), hi(xb, s0, nz0)};
+  o1 = u32x4{lo(ya, s1, nz1), hi(ya, s1, nz1), lo(yb, s1, nz1), hi(yb, s1, nz1)};
+}
+
 // byte N of x as float (v_cvt_f32_ubyteN; the compiler only finds the byte-0 form on its own)
 template <int N>
 __device__ __forceinline__ float ubyte_f32(uint32_t x) {

@@ -431,16 +431,7 @@ int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
   decode_fn fn = pick_decode(a->dtype, pl.use_perm, pl.tn, zp, pl.gm == GM_CHANNEL);
   KParams p = make_kparams(a, pl);
   const int smem = pl.tn == 64 ? DecodeCfg<64>::SMEM : DecodeCfg<128>::SMEM;
-  if (smem > 64 * 1024) {
-    static const void* allowed[32];
-    static int n_allowed = 0;
-    bool seen = false;
-    for (int i = 0; i < n_allowed; ++i) seen |= allowed[i] == (const void*)fn;
-    if (!seen) {
-      W4A16_HIP(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-      if (n_allowed < 32) allowed[n_allowed++] = (const void*)fn;
-    }
-  }
+  W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
   const int64_t grid = (int64_t)pl.tiles * pl.splits;
   if (grid <= 0) return 0;
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(DNW * 64), smem, stream, p);

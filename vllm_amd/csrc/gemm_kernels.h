@@ -1,5 +1,7 @@
 // Kernel parameter block and cross-workgroup helpers shared by the W4A16 GEMM kernels.
 #pragma once
+#include <mutex>
+
 #include "gemm_plan.h"
 
 namespace w4a16 {
@@ -73,6 +75,24 @@ __device__ __forceinline__ f32x4 load_coherent(const float* ptr) {
 __device__ __forceinline__ bool arrive_last(int32_t* counter, int splits) {
   const unsigned old = __builtin_amdgcn_atomic_inc32((unsigned*)counter, (unsigned)(splits - 1), __ATOMIC_RELAXED, "agent");
   return old == (unsigned)(splits - 1);
+}
+
+// Host: more than 64 KiB of dynamic LDS has to be allowed per kernel function; done once per function, device and
+// process (thread-safe).  Returns a HIP error code.
+inline hipError_t allow_dynamic_lds(const void* fn, int bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  struct Key { const void* fn; int dev; };
+  static std::mutex mu;
+  static Key seen[256];
+  static int n_seen = 0;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  for (int i = 0; i < n_seen; ++i)
+    if (seen[i].fn == fn && seen[i].dev == dev) return hipSuccess;
+  if (hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes)) return e;
+  if (n_seen < 256) seen[n_seen++] = Key{fn, dev};
+  return hipSuccess;
 }
 
 // Host: translate the C-ABI arguments and the launch plan into the kernel parameter block.

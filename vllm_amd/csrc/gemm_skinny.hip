@@ -38,16 +38,18 @@ struct SkinnyCfg {
 };
 
 
-template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4>
+template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
+  // ZPF: fp16 zero points laid out like the scales (HQQ); element-wise dequantisation on every tile size
+  static_assert(!ZPF || (DT == DT_F16 && !ZP && GM == GM_GROUPED && !PERM && BITS == 4), "float zero points: fp16 uint4 grouped");
   constexpr int BM = 16 * MB;
   // 8-bit stages hold twice the weight registers: shorter ring
   constexpr int D = (BITS == 8) ? (MB >= 4 ? 2 : 3) : SkinnyCfg<MB>::D;
   constexpr bool UNIT = (GM == GM_CHANNEL);
   // Decode tiles (one m-block) keep the weights as raw magic numbers E+q in the MFMA and apply
   // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
-  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4);
+  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4) && !ZPF;
   constexpr bool HI_TRICK = FOLD && (DT == DT_F16) && !ZP;
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
@@ -143,6 +145,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const int64_t s_row = p.N >> 3;  // u32x4 (8 scales) per scale row; also words per zero-point row
   const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
+  const u32x4* zfp = ZPF ? (const u32x4*)Zp + nt * 8 + c : nullptr;  // fp16 zero points: indexed like the scales
 
   // Activations: lane (row am = l>>2, piece ap = l&3) loads the 16 bytes A[row][32ks + 8ap .. +8), so one
   // 16-lane pass of the load covers 4 rows x 64 contiguous bytes.  The MFMA lane (row m = l&15, g = l>>4)
@@ -156,6 +159,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   struct Stage {
     u32x4 b0, b1, sc;
     u32x4 b0h, b1h;  // 8-bit weights only: second half of the thread's words (w = 2, 3)
+    u32x4 zf;        // float zero points only
     u32x4 a[MB];
     uint32_t zq;
     int gi;
@@ -187,6 +191,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     s.gi = gi;
     if (GM != GM_CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    if (ZPF) s.zf = zfp[(int64_t)gi * s_row];
     s.b0 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks) * b_row);
     s.b1 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks + 1) * b_row);
     if constexpr (BITS == 8) {
@@ -198,7 +203,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   auto dequant_word = [&](const Stage& s, auto w_tag, auto unit_tag, u32x4& o0, u32x4& o1) {
     constexpr int w = decltype(w_tag)::value;
     constexpr bool unit = decltype(unit_tag)::value;
-    if constexpr (BITS == 4) {
+    if constexpr (ZPF) {
+      const uint32_t zs = as_u32(as_h2(s.zf[w]) * as_h2(s.sc[w]));
+      dequant_pair_zpf(s.b0[w], s.b1[w], s.sc[w], zs, o0, o1);
+    } else if constexpr (BITS == 4) {
       uint32_t z0 = 8, z1 = 8;
       if (ZP) {
         z0 = (s.zq >> (4 * w)) & 0xf;
@@ -553,25 +561,23 @@ static int skinny_smem_bytes(int mb) {
   return mb == 1 ? SkinnyCfg<1>::SMEM : mb == 2 ? SkinnyCfg<2>::SMEM : SkinnyCfg<4>::SMEM;
 }
 
+static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
+  switch (mb) {
+    case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, false, 4, true>;
+    case 2: return skinny_kernel<DT_F16, 2, false, GM_GROUPED, false, 4, true>;
+    default: return skinny_kernel<DT_F16, 4, false, GM_GROUPED, false, 4, true>;
+  }
+}
+
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
-  skinny_fn fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
+  skinny_fn fn = (a->flags & W4A16_F_ZP_FLOAT)
+                     ? pick_zpf(pl.mb)
+                     : pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
   if (!fn) return fail(W4A16_EINVAL, "unsupported kernel variant");
   KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);
-  if (smem > 64 * 1024) {
-    // more than 64 KiB of dynamic LDS has to be allowed per kernel function; once per function and process
-    static std::mutex mu;
-    static const void* allowed[64];
-    static int n_allowed = 0;
-    std::lock_guard<std::mutex> lock(mu);
-    bool seen = false;
-    for (int i = 0; i < n_allowed; ++i) seen |= allowed[i] == (const void*)fn;
-    if (!seen) {
-      W4A16_HIP(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-      if (n_allowed < 64) allowed[n_allowed++] = (const void*)fn;
-    }
-  }
+  W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
   const int64_t grid = (int64_t)pl.tiles * pl.splits;
   if (grid <= 0) return 0;
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(NW * 64), smem, stream, p);
