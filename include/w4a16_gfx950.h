@@ -24,13 +24,20 @@ extern "C" {
 enum {
   W4A16_OK = 0,
   W4A16_EINVAL = -1,   /* shape / argument check failed (reference: TORCH_CHECK)     */
-  W4A16_ENOTIMPL = -2, /* valid in the reference, not built here (e.g. 8-bit, fp8)   */
+  W4A16_ENOTIMPL = -2, /* valid in the reference, not built here (e.g. fp4 weights)  */
   W4A16_EHIP = -3      /* a HIP runtime call failed                                  */
 };
 
 /* weight types (decoded from the reference's ScalarType ids by the host layer,
  * vllm/scalar_type.py:136-164, csrc/core/scalar_type.hpp:143-160) */
-enum { W4A16_WTYPE_U4B8 = 0, W4A16_WTYPE_U4 = 1, W4A16_WTYPE_U8B128 = 2 };
+enum {
+  W4A16_WTYPE_U4B8 = 0,
+  W4A16_WTYPE_U4 = 1,
+  W4A16_WTYPE_U8B128 = 2,
+  /* float8_e4m3fn bytes in the 8-bit Marlin layout; b_scales carry the exponent offset the reference folds in at
+     load time (marlin_utils_fp8.py:25-37: x 2^8 for fp16, x 2^120 for bf16); no zero points, no act-order */
+  W4A16_WTYPE_FE4M3 = 3
+};
 /* activation / output / scale element type */
 enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1, W4A16_DTYPE_F32 = 2 /* router logits only */ };
 

@@ -9,6 +9,7 @@ are all part of what is checked:
 
   dequant_marlin(...)   Marlin-layout operands  -> w [K, N] in the activation dtype
   dequant_marlin_float_zp(...)  the same for fp16 zero points (HQQ)
+  dequant_marlin_fp8(...)       the same for float8_e4m3fn weights
   dequant_checkpoint()  GPTQ / AWQ checkpoint   -> w [K, N]   (the CPU baseline path:
                         unpack nibbles, (q-8)*s or (q-z)*s group-broadcast)
   gemm_ref(a, w)        fp32 matmul (+ bias), result in fp32
@@ -87,6 +88,42 @@ def float_zp_test_ref(q, scale, zero, group_size: int):
     b_flat = q.reshape(-1, group_size)
     dequant = (b_flat.to(torch.float16) - zero.reshape(-1, 1)) * scale.reshape(-1, 1)
     return dequant.reshape(n, k).transpose(1, 0).contiguous()
+
+
+def fp8_e4m3fn_table() -> torch.Tensor:
+    """float64 value of each of the 256 float8_e4m3fn codes by the format's closed form (OCP 8-bit float spec,
+    E4M3: bias 7, no infinities, S.1111.111 = NaN): (-1)^s 2^(e-7) (1 + m/8) for e > 0, (-1)^s 2^-6 (m/8) for e = 0.
+    Pinned by (tests/test_oracle_quant.py): literal codes (0x38 = 1, 0x7E = 448, 0x01 = 2^-9, 0x08 = 2^-6,
+    0xC0 = -2) and agreement with torch's own float8_e4m3fn -> float conversion on all 254 finite codes."""
+    vals = []
+    for code in range(256):
+        sgn = -1.0 if code & 0x80 else 1.0
+        e, m = (code >> 3) & 0xF, code & 7
+        if e == 15 and m == 7:
+            vals.append(float("nan"))
+        elif e == 0:
+            vals.append(sgn * 2.0 ** -6 * (m / 8.0))
+        else:
+            vals.append(sgn * 2.0 ** (e - 7) * (1.0 + m / 8.0))
+    return torch.tensor(vals, dtype=torch.float64)
+
+
+def fp8_scale_offset(dtype) -> float:
+    """Factor the reference folds into fp8 Marlin scales at load time (marlin_utils_fp8.py:25-37)."""
+    return 2.0 ** 8 if dtype == torch.float16 else 2.0 ** 120
+
+
+def dequant_marlin_fp8(b_q_weight, b_scales_fused, size_k, size_n, dtype):
+    """fp8 bytes in the 8-bit Marlin layout + Marlin-permuted scales carrying the exponent offset -> dense w[K, N]
+    = fp8.to(dtype) * s evaluated in `dtype` (one rounding), the w_ref of the reference's marlin_quant_fp8_torch
+    (marlin_utils_fp8.py:313-351)."""
+    codes = marlin_unpack_weights8(b_q_weight)
+    assert tuple(codes.shape) == (size_k, size_n)
+    x = fp8_e4m3fn_table()[codes.long()].to(dtype)
+    grouped = b_scales_fused.shape[0] > 1
+    s = marlin_unpermute_scales(b_scales_fused, grouped)
+    s = (s.double() / fp8_scale_offset(dtype)).to(dtype)
+    return x * _expand_groups(s, size_k)
 
 
 def dequant_checkpoint(qweight, scales, qzeros, g_idx, fmt: str, dtype):

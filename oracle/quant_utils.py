@@ -215,3 +215,18 @@ def awq_unpack(packed, num_bits: int = 4) -> torch.Tensor:
     out = np.empty_like(raw).reshape(k, n // pf, pf)
     out[:, :, order] = raw.reshape(k, n // pf, pf)
     return torch.from_numpy(out.reshape(k, n))
+
+
+def quantize_fp8(w: torch.Tensor, group_size: int):
+    """Weight-only fp8 quantizer of the reference's test helper (marlin_utils_fp8.py:313-335), on w [K, N]:
+    scale = absmax / 448 per (group, column) in the weight dtype, codes = (w / scale) cast to float8_e4m3fn
+    (torch's round-to-nearest-even cast), w_ref = codes.to(dtype) * scale.
+    Returns (w_ref [K, N], codes uint8 [K, N], scales [G, N])."""
+    size_k, size_n = w.shape
+    gs = size_k if group_size == -1 else group_size
+    wg = w.t().contiguous().view(size_n, -1, gs)
+    scales = wg.abs().amax(-1) / 448                       # [N, G]
+    rep = scales.repeat_interleave(gs, 1)                  # [N, K]
+    fp8 = (w.t() / rep).to(torch.float8_e4m3fn)
+    w_ref = fp8.to(w.dtype) * rep
+    return w_ref.t().contiguous(), fp8.view(torch.uint8).t().contiguous(), scales.t().contiguous()

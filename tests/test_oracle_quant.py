@@ -245,3 +245,29 @@ def test_float_zp_close_to_the_reference_test_formula():
     s_full, z_full = s.float().repeat_interleave(64, 0), z.float().repeat_interleave(64, 0)
     bound = 2.0 ** -9 * torch.maximum((q.float() * s_full).abs(), (z_full * s_full).abs()) + 1e-7
     assert ((w - ref).abs() <= bound).all()
+
+
+# ------------------------------------------------------------------------------ fp8 weights
+def test_fp8_table_literals_and_torch_conversion():
+    t = gr.fp8_e4m3fn_table()
+    assert t[0x38] == 1.0 and t[0x7E] == 448.0 and t[0x01] == 2.0 ** -9 and t[0x08] == 2.0 ** -6 and t[0xC0] == -2.0
+    assert t[0x00] == 0.0 and t[0x7F].isnan() and t[0xFF].isnan()
+    finite = [c for c in range(256) if c & 0x7F != 0x7F]
+    codes = torch.tensor(finite, dtype=torch.uint8)
+    assert torch.equal(codes.view(torch.float8_e4m3fn).double(), t[codes.long()])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 128])
+def test_fp8_dequant_reproduces_quantizer_w_ref(dtype, group):
+    k, n = 256, 128
+    w = torch.randn(k, n, generator=torch.Generator().manual_seed(21)).to(dtype)
+    w_ref, codes, s = qu.quantize_fp8(w, group)
+    assert codes.dtype == torch.uint8 and s.shape == (1 if group == -1 else k // group, n)
+    assert (codes & 0x7F != 0x7F).all()
+    # |w - w_ref| within half an fp8 step (2^-4 relative) plus the 16-bit roundings
+    assert ((w.float() - w_ref.float()).abs() <= w.float().abs() * 2.0 ** -4 + s.float().repeat_interleave(k // s.shape[0], 0) * 2.0 ** -9).all()
+    mq = ml.marlin_weights_closed_form8(codes.to(torch.int32))
+    ms = ml.marlin_permute_scales(s, k, n, k if group == -1 else group)
+    ms_fused = (ms.double() * gr.fp8_scale_offset(dtype)).to(dtype)
+    assert torch.equal(gr.dequant_marlin_fp8(mq, ms_fused, k, n, dtype), w_ref)

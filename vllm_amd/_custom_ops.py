@@ -91,9 +91,12 @@ def _wtype_code(type_id: int, has_zp: bool) -> int:
     if type_id == scalar_types.uint4.id:
         _check(has_zp, "b_q_type must be uint4b8 or uint8b128 when has_zp = False. Got = uint4")
         return _lib.WTYPE_U4
+    if type_id == scalar_types.float8_e4m3fn.id:
+        _check(not has_zp, "b_q_type must be uint4 or uint8 when has_zp = True. Got = float8_e4m3fn")
+        return _lib.WTYPE_FE4M3
     raise NotImplementedError(
         f"weight type {ScalarType.from_id(type_id)} is not implemented by the gfx950 W4A16 library "
-        "(supported: uint4b8, uint8b128, uint4 with zero points)")
+        "(supported: uint4b8, uint8b128, float8_e4m3fn, uint4 with zero points)")
 
 
 def _pack_factor(type_id: int) -> int:

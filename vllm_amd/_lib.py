@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libw4a16_gfx950.so")
 
 W4A16_OK = 0
-WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128 = 0, 1, 2
+WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128, WTYPE_FE4M3 = 0, 1, 2, 3
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE, F_ZP_FLOAT = 1, 2, 4, 8, 16, 32
 

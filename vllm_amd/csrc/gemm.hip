@@ -18,7 +18,8 @@ static int validate(const w4a16_gemm_args* a) {
               a->struct_size, sizeof(w4a16_gemm_args));
   W4A16_CHECK(a->dtype == W4A16_DTYPE_F16 || a->dtype == W4A16_DTYPE_BF16,
               "gpt_marlin_gemm only supports bfloat16 and float16");
-  W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U4 || a->wtype == W4A16_WTYPE_U8B128,
+  W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U4 || a->wtype == W4A16_WTYPE_U8B128 ||
+                  a->wtype == W4A16_WTYPE_FE4M3,
               "unsupported b_q_type");
   W4A16_CHECK(a->size_m >= 0 && a->size_n > 0 && a->size_k > 0, "bad problem size");
   W4A16_CHECK(a->size_k % 32 == 0, "size_k = %lld is not divisible by 32", (long long)a->size_k);
@@ -34,8 +35,15 @@ static int validate(const w4a16_gemm_args* a) {
   if (has_zp)
     W4A16_CHECK(a->wtype == W4A16_WTYPE_U4, "b_q_type must be uint4 when has_zp = True");
   else
-    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U8B128,
-                "b_q_type must be uint4b8 or uint8b128 when has_zp = False");
+    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3,
+                "b_q_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False");
+  if (a->wtype == W4A16_WTYPE_FE4M3) {
+    // the reference instantiates fp8 weights for channel-wise and group-128 scales without act-order
+    // (csrc/quantization/gptq_marlin/gptq_marlin.cu:266-300 COMMON / BIGGROUP cases); any whole group size is accepted here
+    W4A16_CHECK(a->g_idx == nullptr,
+                "Unsupported shapes: MNK = [%lld, %lld, %lld], has_act_order = 1 with float8_e4m3fn weights",
+                (long long)a->size_m, (long long)a->size_n, (long long)a->size_k);
+  }
   W4A16_CHECK((a->g_idx == nullptr) == (a->perm == nullptr),
               "g_idx and perm must both be given (act-order) or both be empty");
   if (a->flags & W4A16_F_ZP_FLOAT) {
@@ -86,7 +94,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
 
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   // 8-bit weights and float zero points run on the general (skinny) kernel only
-  const bool general_only = a->wtype == W4A16_WTYPE_U8B128 || (a->flags & W4A16_F_ZP_FLOAT) != 0;
+  const bool general_only = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3 ||
+                            (a->flags & W4A16_F_ZP_FLOAT) != 0;
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");

@@ -253,6 +253,45 @@ __device__ __forceinline__ void dequant_pair8(uint32_t xa0, uint32_t xa1, uint32
   }
 }
 
+// fp8 (OCP e4m3fn) weights in the 8-bit Marlin layout.  The scales the op receives carry the exponent offset the
+// reference folds into them at load time (marlin_utils_fp8.py:25-37: s * 2^8 for fp16, s * 2^120 for bf16, because
+// its kernel moves the fp8 bits into the 16-bit format without re-biasing the exponent, dequant.h:320-373).  Here the
+// bytes are converted by v_cvt_pk_f32_fp8 (exact), so the offset is taken out of the scale again (exact, a power of
+// two) and the operand is x * s rounded once to the 16-bit type: the reference's w_ref = fp8.to(dtype) * s.
+template <int DT>
+__device__ __forceinline__ float fp8_scale_unbias() {
+  return (DT == DT_F16) ? 0x1.0p-8f : 0x1.0p-120f;
+}
+template <int DT, bool UNIT_SCALE>
+__device__ __forceinline__ void dequant_pair8_fp8(uint32_t xa0, uint32_t xa1, uint32_t xb0, uint32_t xb1,
+                                                  uint32_t s_pair, u32x4& o0, u32x4& o1) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  float s0 = 1.0f, s1 = 1.0f;
+  if (!UNIT_SCALE) {
+    s0 = ((DT == DT_F16) ? f16_lo_f32(s_pair) : bf16_lo_f32(s_pair)) * fp8_scale_unbias<DT>();
+    s1 = ((DT == DT_F16) ? f16_hi_f32(s_pair) : bf16_hi_f32(s_pair)) * fp8_scale_unbias<DT>();
+  }
+  // a word holds K rows (k0, k0+8, k0+1, k0+9): low half -> (k0, k0+8), high half -> (k0+1, k0+9)
+  auto cvt = [&](uint32_t x, float sf, uint32_t& p_lo, uint32_t& p_hi) {
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)x, false);
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)x, true);
+    if constexpr (DT == DT_F16) {
+      p_lo = pack_f16(a.x * sf, b.x * sf);  // (k0, k0+1)
+      p_hi = pack_f16(a.y * sf, b.y * sf);  // (k0+8, k0+9)
+    } else {
+      p_lo = pack_bf16(a.x * sf, b.x * sf);
+      p_hi = pack_bf16(a.y * sf, b.y * sf);
+    }
+  };
+  uint32_t p0, p1, p2, p3, q0, q1, q2, q3;
+  cvt(xa0, s0, p0, p1);
+  cvt(xb0, s0, p2, p3);
+  cvt(xa1, s1, q0, q1);
+  cvt(xb1, s1, q2, q3);
+  o0 = u32x4{p0, p1, p2, p3};
+  o1 = u32x4{q0, q1, q2, q3};
+}
+
 // "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
 // of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
 // high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the

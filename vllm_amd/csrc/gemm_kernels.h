@@ -136,7 +136,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.top_k = moe ? a->top_k : 1;
   p.mul_topk = moe && (a->flags & W4A16_F_MUL_TOPK_WEIGHTS);
   p.n_sorted = moe ? (int)a->n_sorted : 0;
-  p.b_estride = (a->size_k / 16) * (a->wtype == W4A16_WTYPE_U8B128 ? 4 : 2) * a->size_n;
+  p.b_estride = (a->size_k / 16) * ((a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) ? 4 : 2) * a->size_n;
   p.s_estride = a->num_groups * a->size_n;
   p.z_estride = a->num_groups * (a->size_n / 8);
   p.k_estride = a->size_k;

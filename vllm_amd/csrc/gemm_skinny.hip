@@ -38,10 +38,11 @@ struct SkinnyCfg {
 };
 
 
-template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false>
+template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false, bool FP8 = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
   // ZPF: fp16 zero points laid out like the scales (HQQ); element-wise dequantisation on every tile size
+  static_assert(!FP8 || (BITS == 8 && GM != GM_GIDX && !PERM), "fp8 weights use the 8-bit layout, no act-order");
   static_assert(!ZPF || (DT == DT_F16 && !ZP && GM == GM_GROUPED && !PERM && BITS == 4), "float zero points: fp16 uint4 grouped");
   constexpr int BM = 16 * MB;
   // 8-bit stages hold twice the weight registers: shorter ring
@@ -217,8 +218,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     } else {
       const u32x4& la = (w < 2) ? s.b0 : s.b0h;
       const u32x4& lb = (w < 2) ? s.b1 : s.b1h;
-      dequant_pair8<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
-                              unit ? 0u : s.sc[w], o0, o1);
+      if constexpr (FP8)
+        dequant_pair8_fp8<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
+                                    unit ? 0u : s.sc[w], o0, o1);
+      else
+        dequant_pair8<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
+                                unit ? 0u : s.sc[w], o0, o1);
     }
   };
 
@@ -429,7 +434,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        v[j] *= (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+        v[j] *= ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (FP8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
     }
     if (bias) {
@@ -561,6 +566,21 @@ static int skinny_smem_bytes(int mb) {
   return mb == 1 ? SkinnyCfg<1>::SMEM : mb == 2 ? SkinnyCfg<2>::SMEM : SkinnyCfg<4>::SMEM;
 }
 
+template <int DT>
+static skinny_fn pick_fp8(int mb, int gm) {  // float8_e4m3fn: grouped or channel-wise scales, no act-order
+  switch (mb) {
+    case 1:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, false, 8, false, true>
+                              : skinny_kernel<DT, 1, false, GM_CHANNEL, false, 8, false, true>;
+    case 2:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, false, 8, false, true>
+                              : skinny_kernel<DT, 2, false, GM_CHANNEL, false, 8, false, true>;
+    default:
+      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, false, 8, false, true>
+                              : skinny_kernel<DT, 4, false, GM_CHANNEL, false, 8, false, true>;
+  }
+}
+
 static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
   switch (mb) {
     case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, false, 4, true>;
@@ -571,9 +591,15 @@ static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host:
 
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
-  skinny_fn fn = (a->flags & W4A16_F_ZP_FLOAT)
-                     ? pick_zpf(pl.mb)
-                     : pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
+  skinny_fn fn;
+  if (a->flags & W4A16_F_ZP_FLOAT)
+    fn = pick_zpf(pl.mb);
+  else if (a->wtype == W4A16_WTYPE_FE4M3)
+    fn = (pl.gm == GM_GIDX || pl.use_perm) ? nullptr
+         : a->dtype == DT_F16              ? pick_fp8<DT_F16>(pl.mb, pl.gm)
+                                           : pick_fp8<DT_BF16>(pl.mb, pl.gm);
+  else
+    fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
   if (!fn) return fail(W4A16_EINVAL, "unsupported kernel variant");
   KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);

@@ -27,7 +27,10 @@ def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_ty
     if has_zp is None:
         return (query_marlin_supported_quant_types(False, include_fp_type, device_capability) +
                 query_marlin_supported_quant_types(True, include_fp_type, device_capability))
-    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8, scalar_types.uint8b128]
+    if has_zp:
+        return [scalar_types.uint4]
+    res = [scalar_types.uint4b8, scalar_types.uint8b128]
+    return res + [scalar_types.float8_e4m3fn] if include_fp_type else res
 
 
 def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,

@@ -2,13 +2,15 @@
 
 Host-side mirror of the slice of `ScalarType` (reference vllm/scalar_type.py:136-164, 327-356;
 C++ csrc/core/scalar_type.hpp:120-160) that this path needs: integer types with an optional
-bias.  The id packs, from bit 0 up: exponent:8, mantissa:8, signed:1, bias:32,
+bias, and the 8- and 4-bit float types the ops name (float8_e4m3fn is implemented, float4_e2m1f is recognised).  The id packs, from bit 0 up: exponent:8, mantissa:8, signed:1, bias:32,
 finite_values_only:1, nan_repr:8 — so ids produced by vLLM's own ScalarType decode here and
 vice versa.
 """
 from dataclasses import dataclass
 
+_NAN_REPR_NONE = 0
 _NAN_REPR_IEEE_754 = 1
+_NAN_REPR_EXTD_RANGE_MAX_MIN = 2
 
 
 @dataclass(frozen=True)
@@ -65,7 +67,22 @@ class ScalarType:
     def int_(cls, size_bits: int, bias: int | None) -> "ScalarType":
         return cls(0, size_bits - 1, True, bias or 0)
 
+    @classmethod
+    def float_(cls, exponent: int, mantissa: int, finite_values_only: bool, nan_repr: int) -> "ScalarType":
+        """Non-IEEE float type (scalar_type.py:292-309)."""
+        return cls(exponent, mantissa, True, 0, finite_values_only, nan_repr)
+
+    def is_floating_point(self) -> bool:
+        return self.exponent != 0
+
     def __str__(self) -> str:
+        if self.is_floating_point():
+            s = f"float{self.size_bits}_e{self.exponent}m{self.mantissa}"
+            if self._finite_values_only:
+                s += "f"
+            if self.nan_repr == _NAN_REPR_EXTD_RANGE_MAX_MIN:
+                s += "n"
+            return s
         s = ("int" if self.signed else "uint") + str(self.size_bits)
         return s + (f"b{self.bias}" if self.bias else "")
 
@@ -77,3 +94,5 @@ class scalar_types:
     uint8 = ScalarType.uint(8, None)
     uint4b8 = ScalarType.uint(4, 8)
     uint8b128 = ScalarType.uint(8, 128)
+    float8_e4m3fn = ScalarType.float_(4, 3, True, _NAN_REPR_EXTD_RANGE_MAX_MIN)
+    float4_e2m1f = ScalarType.float_(2, 1, True, _NAN_REPR_NONE)
