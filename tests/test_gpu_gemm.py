@@ -277,3 +277,50 @@ def test_prefill_tail_strips_go_to_the_64_row_kernel(ops, dev, workspace):
     for lo, hi in ((0, 4096), (4096, 6144)):      # prefill-kernel strips, 64-row-kernel strips
         m = gr.error_metrics(out[:, lo:hi], ref[:, lo:hi])
         assert m["max_rel"] <= 4e-2 and m["mean_rel"] < 0.04, (lo, hi, m)
+
+
+# ------------------------------------------------------------ 33..128 rows
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["gptq", "awq", "gptq_act_order", "channel", "gptq_g32"])
+@pytest.mark.parametrize("mnk", [(33, 192, 128), (64, 320, 512), (67, 832, 384), (100, 128, 2048), (128, 4096, 256)])
+def test_rows_33_to_128(ops, dev, workspace, dtype, mode, mnk):
+    """Between the decode and prefill regimes: N/64 odd and even, shallow and deep K (K split or not)."""
+    size_m, size_n, size_k = mnk
+    group = -1 if mode == "channel" else 32 if mode == "gptq_g32" else 128
+    if mode == "gptq_act_order" and size_k == group:
+        pytest.skip("act-order needs more than one group")
+    print(f"rows33-128 {mode} dtype={dtype} m={size_m} n={size_n} k={size_k}", flush=True)
+    layer = make_layer(size_k, size_n, group, dtype, has_zp=(mode == "awq"), act_order=(mode == "gptq_act_order"),
+                       seed=size_m + 1)
+    a = _a(size_m, size_k, dtype, dev, seed=4)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    assert int(workspace.abs().sum()) == 0
+    assert torch.equal(out, run_gemm(ops, layer, a, dev, workspace))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("has_zp", [False, True])
+@pytest.mark.parametrize("group_size", [-1, 64, 128])
+def test_rows_33_to_128_one_hot(ops, dev, workspace, dtype, has_zp, group_size):
+    """Unit-vector rows for 100 rows: wide N with shallow K, narrow N with deep K."""
+    for size_k, size_n in ((256, 1536), (2048, 192)):
+        layer = make_layer(size_k, size_n, group_size, dtype, has_zp=has_zp, seed=9)
+        ks = torch.randperm(size_k, generator=torch.Generator().manual_seed(3))[:100]
+        a = torch.zeros(100, size_k, dtype=dtype)
+        a[torch.arange(100), ks] = 1.0
+        out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+        assert torch.equal(out.cpu(), layer.w_ref[ks])
+
+
+def test_rows_33_to_128_bias_strided_a_given_c(ops, dev, workspace):
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    size_m, size_k, size_n = 90, 1024, 448
+    layer = make_layer(size_k, size_n, 128, torch.bfloat16, has_zp=True, seed=33)
+    g = torch.Generator().manual_seed(34)
+    a = torch.randn(size_m, size_k + 64, generator=g).bfloat16().to(dev)[:, 32:32 + size_k]
+    bias = torch.randn(size_n, generator=g).bfloat16().to(dev)
+    c = torch.full((size_m, size_n), 7.0, dtype=torch.bfloat16, device=dev)
+    out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias), c=c)
+    assert out.data_ptr() == c.data_ptr()
+    check_close(out, a, layer, bias=bias)
