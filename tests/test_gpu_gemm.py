@@ -324,3 +324,19 @@ def test_rows_33_to_128_bias_strided_a_given_c(ops, dev, workspace):
     out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias), c=c)
     assert out.data_ptr() == c.data_ptr()
     check_close(out, a, layer, bias=bias)
+
+
+@pytest.mark.parametrize("ws_len", [64, 128, 256, 1024])
+def test_split_k_with_short_workspaces(ops, dev, ws_len):
+    """K-split launches place the tile counters 1, 2 or 4 ints apart depending on the workspace length (the reference's
+    marlin_make_workspace_new gives one int per compute unit); results do not depend on it and the counters end at zero."""
+    size_m, size_k, size_n = 16, 4096, 4096          # 64 tiles of 64 columns, K split in four
+    layer = make_layer(size_k, size_n, 128, torch.float16, seed=51, rule="absmax7", w_std=0.02)
+    a = _a(size_m, size_k, torch.float16, dev, seed=52)
+    ws = torch.zeros(ws_len, dtype=torch.int32, device=dev)
+    out = run_gemm(ops, layer, a, dev, ws)
+    check_close(out, a, layer)
+    assert int(ws.abs().sum()) == 0
+    big = torch.zeros(4096, dtype=torch.int32, device=dev)
+    assert torch.equal(out, run_gemm(ops, layer, a, dev, big))
+    assert torch.equal(out, run_gemm(ops, layer, a, dev, ws))
