@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define W4A16_ABI_VERSION 1
+#define W4A16_ABI_VERSION 2
 
 enum {
   W4A16_OK = 0,
@@ -36,7 +36,12 @@ enum {
   W4A16_WTYPE_U8B128 = 2,
   /* float8_e4m3fn bytes in the 8-bit Marlin layout; b_scales carry the exponent offset the reference folds in at
      load time (marlin_utils_fp8.py:25-37: x 2^8 for fp16, x 2^120 for bf16); no zero points, no act-order */
-  W4A16_WTYPE_FE4M3 = 3
+  W4A16_WTYPE_FE4M3 = 3,
+  /* float4_e2m1f codes in the 4-bit Marlin layout.  b_scales holds one byte per (group, column) in the order the
+     reference's nvfp4_marlin_process_scales / mxfp4_marlin_process_scales produce
+     (marlin_utils_fp4.py:28-79): group size 16 (NVFP4): scale * 2^7 as unsigned E5M3, with global_scale;
+     group size 32 (MXFP4, bf16 only): E8M0.  No zero points, no act-order, dense op only */
+  W4A16_WTYPE_FE2M1 = 4
 };
 /* activation / output / scale element type */
 enum { W4A16_DTYPE_F16 = 0, W4A16_DTYPE_BF16 = 1, W4A16_DTYPE_F32 = 2 /* router logits only */ };
@@ -101,6 +106,9 @@ typedef struct w4a16_gemm_args {
   int32_t top_k;
   int32_t num_experts;
   int32_t reserved;
+  const void* global_scale;   /* NVFP4 only: one element of the activation type, as the reference's
+                                 nvfp4_marlin_process_global_scale leaves it (marlin_utils_fp4.py:82-93:
+                                 x 2^7 for fp16, x 2^119 for bf16); NULL otherwise            */
 } w4a16_gemm_args;
 
 enum {

@@ -10,6 +10,7 @@ are all part of what is checked:
   dequant_marlin(...)   Marlin-layout operands  -> w [K, N] in the activation dtype
   dequant_marlin_float_zp(...)  the same for fp16 zero points (HQQ)
   dequant_marlin_fp8(...)       the same for float8_e4m3fn weights
+  dequant_marlin_fp4(...)       the same for float4_e2m1f weights (NVFP4 / MXFP4 scale bytes)
   dequant_checkpoint()  GPTQ / AWQ checkpoint   -> w [K, N]   (the CPU baseline path:
                         unpack nibbles, (q-8)*s or (q-z)*s group-broadcast)
   gemm_ref(a, w)        fp32 matmul (+ bias), result in fp32
@@ -124,6 +125,52 @@ def dequant_marlin_fp8(b_q_weight, b_scales_fused, size_k, size_n, dtype):
     s = marlin_unpermute_scales(b_scales_fused, grouped)
     s = (s.double() / fp8_scale_offset(dtype)).to(dtype)
     return x * _expand_groups(s, size_k)
+
+
+FP4_E2M1_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)   # magnitude of codes 0..7; bit 3 is the sign (OCP MX v1.0)
+
+
+def fp4_scale_byte_position(group: int, perm_col: int, size_n: int) -> int:
+    """Flat byte offset, in the processed fp4 scale tensor [G, N], of the scale that sits at (group, perm_col) of
+    the Marlin-permuted scale matrix — closed form of the regrouping in marlin_utils_fp4.py:38-47:
+    rows are taken in pairs; inside a pair the 16 values (row 2i | row 2i+1) of each 8-column chunk are adjacent;
+    inside every run of 4 the middle two are swapped."""
+    chunk, e = perm_col // 8, perm_col % 8
+    pos = (e & 4) | ((e & 1) << 1) | ((e >> 1) & 1)          # (0, 2, 1, 3) applied to the low two bits
+    return (group // 2) * 2 * size_n + chunk * 16 + (group % 2) * 8 + pos
+
+
+def fp4_unprocess_scales(b_scales, fmt: str) -> torch.Tensor:
+    """Processed scale bytes [G, N] (uint8 view) -> true scales float64 [G, N] in Marlin-permuted column order.
+    fmt "nvfp4": byte = high byte of half(s * 2^7) << 1, i.e. s = half(byte << 7) / 2^7;  "mxfp4": s = 2^(byte - 127)."""
+    raw = b_scales.view(torch.uint8)
+    g, n = raw.shape
+    flat = raw.reshape(-1)
+    idx = torch.tensor([[fp4_scale_byte_position(r, c, n) for c in range(n)] for r in range(g)])
+    by = flat[idx].to(torch.int32)
+    if fmt == "nvfp4":
+        return (by << 7).to(torch.int16).view(torch.float16).double() / 128.0
+    return torch.pow(torch.tensor(2.0, dtype=torch.float64), (by - 127).double())
+
+
+def dequant_marlin_fp4(b_q_weight, b_scales, global_scale, size_k, size_n, dtype):
+    """float4_e2m1f codes in the 4-bit Marlin layout + processed scale bytes (+ processed NVFP4 global scale, or None
+    for MXFP4) -> dense w[K, N] = code value * scale * global scale, exact in float64 and rounded once to `dtype`.
+    (The reference's test helper multiplies in `dtype` from left to right, marlin_utils_fp4.py:325-333, which rounds
+    twice: the two agree to one unit in the last place.)
+    Pinned by (tests/test_oracle_quant.py): the code table and byte literals, the closed-form byte position against the
+    restated regrouping, round trips of random scales, and agreement with the test helper's formula to 1 ulp."""
+    codes = marlin_unpack_weights(b_q_weight)
+    assert tuple(codes.shape) == (size_k, size_n)
+    mag = torch.tensor(FP4_E2M1_VALUES, dtype=torch.float64)[(codes & 7).long()]
+    x = torch.where((codes & 8) != 0, -mag, mag)
+    fmt = "nvfp4" if global_scale is not None else "mxfp4"
+    s_perm = fp4_unprocess_scales(b_scales, fmt)
+    s = marlin_unpermute_scales(s_perm, True)
+    gs = 1.0
+    if global_scale is not None:
+        gs = float(global_scale.double().reshape(-1)[0]) / (2.0 ** 7 if dtype == torch.float16 else 2.0 ** 119)
+    return (x * _expand_groups(s, size_k) * gs).to(dtype)
 
 
 def dequant_checkpoint(qweight, scales, qzeros, g_idx, fmt: str, dtype):

@@ -1,0 +1,112 @@
+"""float4_e2m1f weights on gptq_marlin_gemm: NVFP4 (group 16, float8_e4m3fn scales + global scale) and MXFP4
+(group 32, E8M0 scales, bf16), as the reference's test grid feeds them
+(tests/kernels/quantization/test_marlin_gemm.py:262-277 via rand_marlin_weight_{nvfp4,mxfp4}_like)."""
+import pytest
+import torch
+
+from oracle import gemm_ref as gr
+
+pytestmark = pytest.mark.gpu
+
+MNK_FACTORS = [(1, 1, 1), (1, 4, 8), (1, 7, 5), (13, 17, 67), (26, 37, 13), (67, 13, 11), (257, 13, 11), (658, 13, 11)]
+TOL = {torch.float16: 2e-2, torch.bfloat16: 4e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import vllm_amd.ops as o
+    return o
+
+
+@pytest.fixture(scope="module")
+def workspace(dev):
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    return marlin_make_workspace_new(dev)
+
+
+def make(kind, size_k, size_n, dtype, dev, seed):
+    """Operands from the host mirror of the reference's random-weight helpers; w from the oracle's decode of the very
+    tensors the op receives."""
+    from vllm_amd import marlin_utils_fp4 as f4
+    torch.manual_seed(seed)
+    weight = torch.randn(size_n, size_k, dtype=dtype, device=dev)
+    if kind == "nvfp4":
+        w_helper, mq, ms, gs = f4.rand_marlin_weight_nvfp4_like(weight, 16)
+    else:
+        w_helper, mq, ms = f4.rand_marlin_weight_mxfp4_like(weight, 32)
+        gs = None
+    w = gr.dequant_marlin_fp4(mq.cpu(), ms.cpu().view(torch.uint8), None if gs is None else gs.cpu().view(1), size_k, size_n,
+                              dtype)
+    return w, w_helper, mq, ms, None if gs is None else gs.view(1)
+
+
+def run(ops, a, mq, ms, gs, workspace, size_n, size_k, bias=None):
+    import vllm_amd.scalar_type as vst
+    return ops.gptq_marlin_gemm(a, None, mq, bias, ms, gs, None, None, None, workspace, vst.scalar_types.float4_e2m1f,
+                                a.shape[0], size_n, size_k, is_k_full=True, use_fp32_reduce=True)
+
+
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("nvfp4", torch.bfloat16), ("mxfp4", torch.bfloat16)])
+@pytest.mark.parametrize("size_m", [1, 16, 40])
+def test_one_hot_rows_reproduce_the_decoded_weights(ops, dev, workspace, kind, dtype, size_m):
+    size_k, size_n = 256, 192
+    w, w_helper, mq, ms, gs = make(kind, size_k, size_n, dtype, dev, 3)
+    # the helper's left-to-right product rounds twice: within one unit in the last place of the oracle
+    assert ((w.double() - w_helper.cpu().double()).abs() <= w.double().abs() * torch.finfo(dtype).eps).all()
+    rows = torch.randperm(size_k, generator=torch.Generator().manual_seed(size_m))[:size_m]
+    a = torch.zeros(size_m, size_k, dtype=dtype)
+    a[torch.arange(size_m), rows] = 1.0
+    out = run(ops, a.to(dev), mq, ms, gs, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("nvfp4", torch.bfloat16), ("mxfp4", torch.bfloat16)])
+@pytest.mark.parametrize("n_chunk", [64, 256])
+@pytest.mark.parametrize("mnk", MNK_FACTORS)
+def test_reference_grid(ops, dev, workspace, kind, dtype, n_chunk, mnk):
+    mf, nf, kf = mnk
+    size_m, size_k, size_n = mf, 128 * kf, n_chunk * nf
+    print(f"fp4 grid {kind} dtype={dtype} m={size_m} n={size_n} k={size_k}", flush=True)
+    w, w_helper, mq, ms, gs = make(kind, size_k, size_n, dtype, dev, 11 + mf)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).to(dtype)
+    out = run(ops, a.to(dev), mq, ms, gs, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w))
+    assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
+    # the reference's own check: mean|d| / mean|ref| < 0.04 against matmul(a, w_ref) of the helper
+    ref = torch.matmul(a.float(), w_helper.cpu().float())
+    assert float((out.float() - ref).abs().mean() / ref.abs().mean()) < 0.04
+
+
+def test_linear_helpers_and_bias(ops, dev, workspace):
+    from vllm_amd import marlin_utils_fp4 as f4
+    from vllm_amd.marlin_utils import marlin_permute_bias
+    size_k, size_n = 512, 256
+    for kind, dtype in (("nvfp4", torch.float16), ("mxfp4", torch.bfloat16)):
+        w, _, mq, ms, gs = make(kind, size_k, size_n, dtype, dev, 6)
+        x = torch.randn(2, 5, size_k, generator=torch.Generator().manual_seed(7)).to(dtype)
+        bias = torch.randn(size_n, generator=torch.Generator().manual_seed(8)).to(dtype)
+        out = f4.apply_fp4_marlin_linear(x.to(dev), mq, ms, gs, workspace, size_n, size_k, marlin_permute_bias(bias.to(dev)))
+        assert out.shape == (2, 5, size_n)
+        m = gr.error_metrics(out.cpu().view(10, size_n), gr.gemm_ref(x.view(10, size_k), w, bias))
+        assert m["max_rel"] <= TOL[dtype], m
+
+
+def test_argument_errors(ops, dev, workspace):
+    import vllm_amd.scalar_type as vst
+    size_k, size_n = 256, 128
+    _, _, mq, ms, gs = make("nvfp4", size_k, size_n, torch.float16, dev, 9)
+    a = torch.randn(4, size_k).half().to(dev)
+    fp4 = vst.scalar_types.float4_e2m1f
+    with pytest.raises(RuntimeError, match="global_scale parameter must be passed"):
+        ops.gptq_marlin_gemm(a, None, mq, None, ms, None, None, None, None, workspace, fp4, 4, size_n, size_k)
+    with pytest.raises(RuntimeError, match="b_scales must be"):
+        ops.gptq_marlin_gemm(a, None, mq, None, ms.view(torch.uint8).half(), gs, None, None, None, workspace, fp4, 4,
+                             size_n, size_k)
+    _, _, mq2, ms2, _ = make("mxfp4", size_k, size_n, torch.bfloat16, dev, 9)
+    with pytest.raises(RuntimeError, match="bfloat16"):       # MXFP4 with fp16 activations
+        ops.gptq_marlin_gemm(a, None, mq2, None, ms2, None, None, None, None, workspace, fp4, 4, size_n, size_k)
+    with pytest.raises(RuntimeError, match="only be used for nvfp4"):
+        ops.gptq_marlin_gemm(a.bfloat16(), None, mq2, None, ms2, gs.bfloat16(), None, None, None, workspace, fp4, 4,
+                             size_n, size_k)
+    assert int(workspace.abs().sum()) == 0

@@ -74,7 +74,7 @@ def test_shape_gates():
     assert not ok and "group_size" in why
     from vllm_amd.scalar_type import scalar_types
     assert mu.query_marlin_supported_quant_types(False) == [scalar_types.uint4b8, scalar_types.uint8b128,
-                                                            scalar_types.float8_e4m3fn]
+                                                            scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f]
     assert mu.query_marlin_supported_quant_types(False, include_fp_type=False) == [scalar_types.uint4b8,
                                                                                    scalar_types.uint8b128]
     assert mu.query_marlin_supported_quant_types(True) == [scalar_types.uint4]

@@ -271,3 +271,75 @@ def test_fp8_dequant_reproduces_quantizer_w_ref(dtype, group):
     ms = ml.marlin_permute_scales(s, k, n, k if group == -1 else group)
     ms_fused = (ms.double() * gr.fp8_scale_offset(dtype)).to(dtype)
     assert torch.equal(gr.dequant_marlin_fp8(mq, ms_fused, k, n, dtype), w_ref)
+
+
+# ------------------------------------------------------------------------------ fp4 weights
+def _regroup_restated(t):
+    """The reference's regrouping of a Marlin-permuted [G, N] tensor, restated with its own tensor ops
+    (marlin_utils_fp4.py:38-47), as the thing the closed-form byte position is checked against."""
+    g, n = t.shape
+    t = t.view(g // 2, 2, -1, 8).permute(0, 2, 1, 3).reshape(g, n)
+    return t.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(g, n)
+
+
+def test_fp4_code_table_and_scale_byte_literals():
+    assert gr.FP4_E2M1_VALUES == (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
+    # NVFP4 scale byte: high byte of half(s * 2^7) << 1.  1.0 -> half(128) = 0x5800 -> 0xB0; 448 -> 0x7B00 -> 0xF6;
+    # 2^-9 -> half(2^-2) = 0x3400 -> 0x68
+    for s, byte in ((1.0, 0xB0), (448.0, 0xF6), (2.0 ** -9, 0x68), (0.5, 0xA8)):
+        raw = torch.tensor([[byte] * 8] * 2, dtype=torch.uint8)
+        assert torch.all(gr.fp4_unprocess_scales(raw, "nvfp4") == s)
+    raw = torch.tensor([[127, 100, 120, 130] * 2] * 2, dtype=torch.uint8)
+    got = gr.fp4_unprocess_scales(raw, "mxfp4")
+    assert set(got.flatten().tolist()) == {1.0, 2.0 ** -27, 2.0 ** -7, 8.0}
+
+
+def test_fp4_scale_byte_position_matches_the_regrouping():
+    g, n = 6, 128
+    ident = torch.arange(g * n, dtype=torch.int32).view(g, n)         # value = flat index in the permuted matrix
+    out = _regroup_restated(ident).reshape(-1)
+    for r in range(g):
+        for c in range(n):
+            assert int(out[gr.fp4_scale_byte_position(r, c, n)]) == r * n + c
+    # hand-derived: rows 2, 3 (second pair), permuted column 8*5 + 3 of row 3: pair offset 2n*1, chunk 5 -> 80,
+    # second row of the pair -> +8, element 3 of (0,2,1,3)-swapped run -> position 3
+    assert gr.fp4_scale_byte_position(3, 43, n) == 2 * n + 80 + 8 + 3
+    assert gr.fp4_scale_byte_position(0, 1, n) == 2 and gr.fp4_scale_byte_position(0, 2, n) == 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_nvfp4_dequant_against_the_test_helper_formula(dtype):
+    """w = value * global_scale * scale evaluated left to right in `dtype` (the reference helper's w_ref) agrees with
+    the single-rounding oracle to one unit in the last place, and exactly when the global scale is a power of two."""
+    k, n, group = 128, 64, 16
+    g = torch.Generator().manual_seed(31)
+    codes = torch.randint(0, 16, (k, n), generator=g, dtype=torch.int32)
+    scales = (torch.rand(k // group, n, generator=g) * 4 + 0.01).to(torch.float8_e4m3fn)
+    table = torch.tensor(gr.FP4_E2M1_VALUES + tuple(-v for v in gr.FP4_E2M1_VALUES), dtype=dtype)
+    mq = ml.gptq_marlin_repack(qu.gptq_pack(codes), None, k, n)
+    ms = ml.marlin_permute_scales(scales.to(dtype), k, n, group)
+    byts = ((_regroup_restated(ms.to(torch.half)) * 128).view(torch.int16) << 1).view(torch.uint8)[:, 1::2].contiguous()
+    for gs_val in (0.25, 0.0123):
+        gs = torch.tensor(gs_val, dtype=dtype)
+        gs_proc = (gs.double() * (2.0 ** 7 if dtype == torch.float16 else 2.0 ** 119)).to(dtype).view(1)
+        w = gr.dequant_marlin_fp4(mq, byts, gs_proc, k, n, dtype)
+        helper = table[codes.long()] * gs * scales.to(dtype).repeat_interleave(group, 0)
+        if gs_val == 0.25:
+            assert torch.equal(w, helper)
+        else:
+            ulp = torch.finfo(dtype).eps
+            assert ((w.double() - helper.double()).abs() <= helper.double().abs() * ulp).all()
+
+
+def test_mxfp4_dequant_is_exact():
+    k, n, group = 128, 128, 32
+    g = torch.Generator().manual_seed(32)
+    codes = torch.randint(0, 16, (k, n), generator=g, dtype=torch.int32)
+    sbytes = torch.randint(100, 125, (k // group, n), generator=g, dtype=torch.uint8)
+    scales = sbytes.view(torch.float8_e8m0fnu).to(torch.bfloat16)
+    table = torch.tensor(gr.FP4_E2M1_VALUES + tuple(-v for v in gr.FP4_E2M1_VALUES), dtype=torch.bfloat16)
+    mq = ml.gptq_marlin_repack(qu.gptq_pack(codes), None, k, n)
+    ms = ml.marlin_permute_scales(scales, k, n, group)
+    byts = _regroup_restated(ms).to(torch.float8_e8m0fnu).view(torch.uint8)
+    w = gr.dequant_marlin_fp4(mq, byts, None, k, n, torch.bfloat16)
+    assert torch.equal(w, table[codes.long()] * scales.repeat_interleave(group, 0))

@@ -94,9 +94,12 @@ def _wtype_code(type_id: int, has_zp: bool) -> int:
     if type_id == scalar_types.float8_e4m3fn.id:
         _check(not has_zp, "b_q_type must be uint4 or uint8 when has_zp = True. Got = float8_e4m3fn")
         return _lib.WTYPE_FE4M3
+    if type_id == scalar_types.float4_e2m1f.id:
+        _check(not has_zp, "b_q_type must be uint4 or uint8 when has_zp = True. Got = float4_e2m1f")
+        return _lib.WTYPE_FE2M1
     raise NotImplementedError(
         f"weight type {ScalarType.from_id(type_id)} is not implemented by the gfx950 W4A16 library "
-        "(supported: uint4b8, uint8b128, float8_e4m3fn, uint4 with zero points)")
+        "(supported: uint4b8, uint8b128, float8_e4m3fn, float4_e2m1f, uint4 with zero points)")
 
 
 def _pack_factor(type_id: int) -> int:
@@ -213,10 +216,26 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
     _check(b_scales.is_cuda and b_scales.is_contiguous(), "b_scales is not a contiguous GPU tensor")
     _check(b_scales.dim() == 2 and b_scales.size(1) == size_n,
            f"b_scales dim 1 = {b_scales.size(-1)} is not size_n = {size_n}")
-    _check(b_scales.dtype == a.dtype, "scalar type of a and b_scales must match")
-    _check(_opt(global_scale) is None, "global_scale can only be used for nvfp4 format.")
-    _check(workspace.is_cuda and workspace.dtype == torch.int32, "workspace must be an int32 GPU tensor")
     num_groups = b_scales.size(0)
+    is_fp4 = int(b_q_type) == scalar_types.float4_e2m1f.id
+    gscale = _opt(global_scale)
+    if is_fp4:
+        # one byte per (group, column): NVFP4 (group 16) float8_e4m3fn + global_scale, MXFP4 (group 32) float8_e8m0fnu
+        group_size = size_k // num_groups if num_groups > 0 and size_k % num_groups == 0 else 0
+        _check(group_size in (16, 32),
+               "float4_e2m1f only supports group_size == 16 (NVFP4) and group_size == 32 (MXFP4)")
+        want = torch.float8_e4m3fn if group_size == 16 else torch.float8_e8m0fnu
+        _check(b_scales.dtype == want, f"b_scales must be {want} for float4_e2m1f with group_size = {group_size}")
+        if group_size == 16:
+            _check(gscale is not None, "the global_scale parameter must be passed for nvfp4 format.")
+            _check(gscale.is_cuda and gscale.numel() == 1 and gscale.dtype == a.dtype,
+                   "global_scale must be one element of the activation type on the GPU")
+        else:
+            _check(gscale is None, "global_scale can only be used for nvfp4 format.")
+    else:
+        _check(b_scales.dtype == a.dtype, "scalar type of a and b_scales must match")
+        _check(gscale is None, "global_scale can only be used for nvfp4 format.")
+    _check(workspace.is_cuda and workspace.dtype == torch.int32, "workspace must be an int32 GPU tensor")
 
     g_idx, perm = _opt(g_idx_or_none), _opt(perm_or_none)
     _check((g_idx is None) == (perm is None),
@@ -268,6 +287,7 @@ def _gptq_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, g
     args = _lib.GemmArgs()
     _fill_common(args, a, c, b_q_weight, b_bias, b_scales, b_zeros, g_idx, perm, workspace, wtype,
                  size_m, size_n, size_k, num_groups, flags)
+    args.global_scale = None if gscale is None else gscale.data_ptr()
     _run_gemm(args, a.device)
     return c
 

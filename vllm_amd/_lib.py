@@ -10,8 +10,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libw4a16_gfx950.so")
 
 W4A16_OK = 0
-WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128, WTYPE_FE4M3 = 0, 1, 2, 3
+WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128, WTYPE_FE4M3, WTYPE_FE2M1 = 0, 1, 2, 3, 4
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
+ABI_VERSION = 2  # W4A16_ABI_VERSION of include/w4a16_gfx950.h this mirror was written against
 F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE, F_ZP_FLOAT = 1, 2, 4, 8, 16, 32
 
 c_void_p, c_i64, c_i32, c_u32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32
@@ -29,7 +30,7 @@ class GemmArgs(ctypes.Structure):
         ("sorted_token_ids", c_void_p), ("expert_ids", c_void_p),
         ("num_tokens_past_padded", c_void_p), ("topk_weights", c_void_p),
         ("n_sorted", c_i64), ("moe_block_size", c_i32), ("top_k", c_i32),
-        ("num_experts", c_i32), ("reserved", c_i32),
+        ("num_experts", c_i32), ("reserved", c_i32), ("global_scale", c_void_p),
     ]
 
 
@@ -64,7 +65,7 @@ def load() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
-        if lib.w4a16_abi_version() != 1:
+        if lib.w4a16_abi_version() != ABI_VERSION:
             raise ImportError("w4a16 ABI version mismatch")
         _lib = lib
     return _lib

@@ -19,7 +19,7 @@ static int validate(const w4a16_gemm_args* a) {
   W4A16_CHECK(a->dtype == W4A16_DTYPE_F16 || a->dtype == W4A16_DTYPE_BF16,
               "gpt_marlin_gemm only supports bfloat16 and float16");
   W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U4 || a->wtype == W4A16_WTYPE_U8B128 ||
-                  a->wtype == W4A16_WTYPE_FE4M3,
+                  a->wtype == W4A16_WTYPE_FE4M3 || a->wtype == W4A16_WTYPE_FE2M1,
               "unsupported b_q_type");
   W4A16_CHECK(a->size_m >= 0 && a->size_n > 0 && a->size_k > 0, "bad problem size");
   W4A16_CHECK(a->size_k % 32 == 0, "size_k = %lld is not divisible by 32", (long long)a->size_k);
@@ -35,8 +35,26 @@ static int validate(const w4a16_gemm_args* a) {
   if (has_zp)
     W4A16_CHECK(a->wtype == W4A16_WTYPE_U4, "b_q_type must be uint4 when has_zp = True");
   else
-    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3,
-                "b_q_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False");
+    W4A16_CHECK(a->wtype == W4A16_WTYPE_U4B8 || a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3 ||
+                    a->wtype == W4A16_WTYPE_FE2M1,
+                "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False");
+  if (a->wtype == W4A16_WTYPE_FE2M1) {
+    if (a->flags & W4A16_F_MOE)
+      return fail(W4A16_ENOTIMPL, "float4_e2m1f weights are not implemented for the MoE op in this build");
+    const int64_t gs = a->num_groups > 0 && a->size_k % a->num_groups == 0 ? a->size_k / a->num_groups : 0;
+    W4A16_CHECK(gs == 16 || gs == 32, "float4_e2m1f only supports group_size == 16 (NVFP4) and group_size == 32 (MXFP4)");
+    W4A16_CHECK(a->g_idx == nullptr, "Unsupported shapes: act-order with float4_e2m1f weights");
+    // scale bytes of two k-tiles (NVFP4) or two k-steps (MXFP4) are interleaved: whole pairs only
+    W4A16_CHECK(a->num_groups % 2 == 0, "float4_e2m1f: the number of scale groups must be even");
+    if (gs == 16)
+      W4A16_CHECK(a->global_scale != nullptr, "the global_scale parameter must be passed for nvfp4 format.");
+    else
+      W4A16_CHECK(a->global_scale == nullptr, "global_scale can only be used for nvfp4 format.");
+    if (gs == 32)
+      W4A16_CHECK(a->dtype == W4A16_DTYPE_BF16, "MXFP4 (group_size == 32) needs bfloat16 activations");
+  } else {
+    W4A16_CHECK(a->global_scale == nullptr, "global_scale can only be used for nvfp4 format.");
+  }
   if (a->wtype == W4A16_WTYPE_FE4M3) {
     // the reference instantiates fp8 weights for channel-wise and group-128 scales without act-order
     // (csrc/quantization/gptq_marlin/gptq_marlin.cu:266-300 COMMON / BIGGROUP cases); any whole group size is accepted here
@@ -80,6 +98,10 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   if (act_order && !k_full) {
     W4A16_CHECK(a->b_zeros == nullptr, "act-order with partial groups does not support zero points");
     pl.gm = GM_GIDX;
+  } else if (a->wtype == W4A16_WTYPE_FE2M1) {
+    // one 16-byte scale record per lane and k-step (NVFP4: its two k-tiles) or per two k-steps (MXFP4)
+    pl.gm = GM_GROUPED;
+    pl.group_ksteps = a->size_k / a->num_groups == 16 ? 1 : 2;
   } else if (a->num_groups > 1) {
     W4A16_CHECK(a->size_k % a->num_groups == 0, "size_k = %lld, is not divisible by b_scales.size(0) = %lld",
                 (long long)a->size_k, (long long)a->num_groups);
@@ -95,6 +117,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   // 8-bit weights and float zero points run on the general (skinny) kernel only
   const bool general_only = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3 ||
+                            a->wtype == W4A16_WTYPE_FE2M1 ||
                             (a->flags & W4A16_F_ZP_FLOAT) != 0;
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)

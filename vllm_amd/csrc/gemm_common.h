@@ -292,6 +292,45 @@ __device__ __forceinline__ void dequant_pair8_fp8(uint32_t xa0, uint32_t xa1, ui
   o1 = u32x4{q0, q1, q2, q3};
 }
 
+// fp4 (float4_e2m1f) weights in the 4-bit Marlin layout.  A byte of a Marlin word holds the codes of K rows (k0, k0+8)
+// [bytes 0, 1: columns n0, n0+8] or (k0+1, k0+9) [bytes 2, 3]; v_cvt_scalef32_pk_f32_fp4 turns one byte into two exact
+// fp32 values.  sa* / sb*: true scales (fp32) of k-tile a / b for column half 0 / 1; x * s has at most 6 significant
+// bits, so the operand is exact in either 16-bit type.
+template <int DT>
+__device__ __forceinline__ void dequant_pair_fp4(uint32_t xa, uint32_t xb, float sa0, float sa1, float sb0, float sb1,
+                                                 u32x4& o0, u32x4& o1) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  auto pack = [](float lo, float hi) { return DT == DT_F16 ? pack_f16(lo, hi) : pack_bf16(lo, hi); };
+  auto tile = [&](uint32_t x, float s0, float s1, uint32_t& p0_lo, uint32_t& p0_hi, uint32_t& p1_lo, uint32_t& p1_hi) {
+    const f32x2 c0a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, 0);  // column n0:   (k0, k0+8)
+    const f32x2 c1a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, 1);  // column n0+8: (k0, k0+8)
+    const f32x2 c0b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, 2);  // column n0:   (k0+1, k0+9)
+    const f32x2 c1b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, 3);  // column n0+8: (k0+1, k0+9)
+    p0_lo = pack(c0a.x * s0, c0b.x * s0);  // (k0, k0+1)
+    p0_hi = pack(c0a.y * s0, c0b.y * s0);  // (k0+8, k0+9)
+    p1_lo = pack(c1a.x * s1, c1b.x * s1);
+    p1_hi = pack(c1a.y * s1, c1b.y * s1);
+  };
+  uint32_t p0, p1, p2, p3, q0, q1, q2, q3;
+  tile(xa, sa0, sa1, p0, p1, q0, q1);
+  tile(xb, sb0, sb1, p2, p3, q2, q3);
+  o0 = u32x4{p0, p1, p2, p3};
+  o1 = u32x4{q0, q1, q2, q3};
+}
+// Scale bytes of Marlin word w in a lane's 16-byte fp4 scale record: 8 bytes per k-tile (NVFP4) or k-step (MXFP4),
+// stored in the order (e0, e2, e1, e3, e4, e6, e5, e7) with e = 2w + half (marlin_utils_fp4.py:44-47, 68-71).
+// half_rec: the 8 bytes as two dwords; returns byte of column half 0 in bits 0..7 and of half 1 in bits 16..23.
+__device__ __forceinline__ uint32_t fp4_scale_bytes(uint32_t d_lo, uint32_t d_hi, int w) {
+  const uint32_t d = (w >> 1) ? d_hi : d_lo;
+  return (d >> (8 * (w & 1))) & 0x00ff00ffu;
+}
+// NVFP4 scale byte -> fp32: the byte is the top byte of half(s * 2^7) << 1 (unsigned E5M3)
+__device__ __forceinline__ float nvfp4_scale_f32(uint32_t byte) {
+  return f16_lo_f32(byte << 7) * 0x1.0p-7f;
+}
+// MXFP4 scale byte (E8M0) -> fp32: 2^(b - 127)
+__device__ __forceinline__ float mxfp4_scale_f32(uint32_t byte) { return __builtin_bit_cast(float, byte << 23); }
+
 // "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
 // of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
 // high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the

@@ -16,6 +16,7 @@ struct KParams {
   const int32_t* gidx;
   const int32_t* perm;
   const void* bias;
+  const void* gscale;  // NVFP4 global scale (one element of the activation type), else null
   float* ctmp;
   int32_t* locks;
   int lock_stride;
@@ -108,6 +109,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.gidx = pl.gm == GM_GIDX ? a->g_idx : nullptr;
   p.perm = pl.use_perm ? a->perm : nullptr;
   p.bias = a->b_bias;
+  p.gscale = a->global_scale;
   p.ctmp = a->c_tmp;
   p.locks = a->workspace;
   // counters of neighbouring tiles 16 bytes apart when the workspace is long enough (arrivals complete sooner)

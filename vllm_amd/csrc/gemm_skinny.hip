@@ -38,10 +38,12 @@ struct SkinnyCfg {
 };
 
 
-template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false, bool FP8 = false>
+// FP4: 0 = integer weights, 1 = float4_e2m1f with NVFP4 scales (per k-tile), 2 = with MXFP4 scales (per k-step)
+template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false, bool FP8 = false, int FP4 = 0>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
   // ZPF: fp16 zero points laid out like the scales (HQQ); element-wise dequantisation on every tile size
+  static_assert(FP4 == 0 || (BITS == 4 && !ZP && !ZPF && GM == GM_GROUPED && !PERM), "fp4 weights: grouped scale records");
   static_assert(!FP8 || (BITS == 8 && GM != GM_GIDX && !PERM), "fp8 weights use the 8-bit layout, no act-order");
   static_assert(!ZPF || (DT == DT_F16 && !ZP && GM == GM_GROUPED && !PERM && BITS == 4), "float zero points: fp16 uint4 grouped");
   constexpr int BM = 16 * MB;
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   constexpr bool UNIT = (GM == GM_CHANNEL);
   // Decode tiles (one m-block) keep the weights as raw magic numbers E+q in the MFMA and apply
   // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
-  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4) && !ZPF;
+  constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4) && !ZPF && FP4 == 0;
   constexpr bool HI_TRICK = FOLD && (DT == DT_F16) && !ZP;
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
@@ -193,6 +195,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     if (GM != GM_CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     if (ZPF) s.zf = zfp[(int64_t)gi * s_row];
+    if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
     s.b0 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks) * b_row);
     s.b1 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks + 1) * b_row);
     if constexpr (BITS == 8) {
@@ -204,7 +207,15 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   auto dequant_word = [&](const Stage& s, auto w_tag, auto unit_tag, u32x4& o0, u32x4& o1) {
     constexpr int w = decltype(w_tag)::value;
     constexpr bool unit = decltype(unit_tag)::value;
-    if constexpr (ZPF) {
+    if constexpr (FP4 == 1) {
+      const uint32_t ba = fp4_scale_bytes(s.sc[0], s.sc[1], w), bb = fp4_scale_bytes(s.sc[2], s.sc[3], w);
+      dequant_pair_fp4<DT>(s.b0[w], s.b1[w], nvfp4_scale_f32(ba & 0xff), nvfp4_scale_f32(ba >> 16),
+                           nvfp4_scale_f32(bb & 0xff), nvfp4_scale_f32(bb >> 16), o0, o1);
+    } else if constexpr (FP4 == 2) {
+      const uint32_t bs = s.zq ? fp4_scale_bytes(s.sc[2], s.sc[3], w) : fp4_scale_bytes(s.sc[0], s.sc[1], w);
+      const float s0 = mxfp4_scale_f32(bs & 0xff), s1 = mxfp4_scale_f32(bs >> 16);
+      dequant_pair_fp4<DT>(s.b0[w], s.b1[w], s0, s1, s0, s1, o0, o1);
+    } else if constexpr (ZPF) {
       const uint32_t zs = as_u32(as_h2(s.zf[w]) * as_h2(s.sc[w]));
       dequant_pair_zpf(s.b0[w], s.b1[w], s.sc[w], zs, o0, o1);
     } else if constexpr (BITS == 4) {
@@ -437,6 +448,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
         v[j] *= ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (FP8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
     }
+    if constexpr (FP4 == 1) {
+      // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
+      const uint16_t gv = *(const uint16_t*)p.gscale;
+      const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] *= gs;
+    }
     if (bias) {
       const int base = ncol & ~31, cl = ncol & 31;
 #pragma unroll
@@ -581,6 +599,15 @@ static skinny_fn pick_fp8(int mb, int gm) {  // float8_e4m3fn: grouped or channe
   }
 }
 
+template <int DT, int FP4>
+static skinny_fn pick_fp4(int mb) {  // float4_e2m1f (validated on the host: grouped records, no act-order, dense)
+  switch (mb) {
+    case 1: return skinny_kernel<DT, 1, false, GM_GROUPED, false, 4, false, false, FP4>;
+    case 2: return skinny_kernel<DT, 2, false, GM_GROUPED, false, 4, false, false, FP4>;
+    default: return skinny_kernel<DT, 4, false, GM_GROUPED, false, 4, false, false, FP4>;
+  }
+}
+
 static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
   switch (mb) {
     case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, false, 4, true>;
@@ -594,6 +621,9 @@ int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
   skinny_fn fn;
   if (a->flags & W4A16_F_ZP_FLOAT)
     fn = pick_zpf(pl.mb);
+  else if (a->wtype == W4A16_WTYPE_FE2M1)
+    fn = a->global_scale ? (a->dtype == DT_F16 ? pick_fp4<DT_F16, 1>(pl.mb) : pick_fp4<DT_BF16, 1>(pl.mb))
+                         : pick_fp4<DT_BF16, 2>(pl.mb);
   else if (a->wtype == W4A16_WTYPE_FE4M3)
     fn = (pl.gm == GM_GIDX || pl.use_perm) ? nullptr
          : a->dtype == DT_F16              ? pick_fp8<DT_F16>(pl.mb, pl.gm)

@@ -30,7 +30,7 @@ def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_ty
     if has_zp:
         return [scalar_types.uint4]
     res = [scalar_types.uint4b8, scalar_types.uint8b128]
-    return res + [scalar_types.float8_e4m3fn] if include_fp_type else res
+    return res + [scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f] if include_fp_type else res
 
 
 def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,
