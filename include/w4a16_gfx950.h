@@ -40,7 +40,7 @@ enum {
   /* float4_e2m1f codes in the 4-bit Marlin layout.  b_scales holds one byte per (group, column) in the order the
      reference's nvfp4_marlin_process_scales / mxfp4_marlin_process_scales produce
      (marlin_utils_fp4.py:28-79): group size 16 (NVFP4): scale * 2^7 as unsigned E5M3, with global_scale;
-     group size 32 (MXFP4, bf16 only): E8M0.  No zero points, no act-order, dense op only */
+     group size 32 (MXFP4, bf16 only): E8M0.  No zero points, no act-order */
   W4A16_WTYPE_FE2M1 = 4
 };
 /* activation / output / scale element type */
@@ -106,7 +106,7 @@ typedef struct w4a16_gemm_args {
   int32_t top_k;
   int32_t num_experts;
   int32_t reserved;
-  const void* global_scale;   /* NVFP4 only: one element of the activation type, as the reference's
+  const void* global_scale;   /* NVFP4 only: [E,] one element of the activation type, as the reference's
                                  nvfp4_marlin_process_global_scale leaves it (marlin_utils_fp4.py:82-93:
                                  x 2^7 for fp16, x 2^119 for bf16); NULL otherwise            */
 } w4a16_gemm_args;

@@ -110,3 +110,31 @@ def test_argument_errors(ops, dev, workspace):
         ops.gptq_marlin_gemm(a.bfloat16(), None, mq2, None, ms2, gs.bfloat16(), None, None, None, workspace, fp4, 4,
                              size_n, size_k)
     assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("nvfp4", torch.bfloat16), ("mxfp4", torch.bfloat16)])
+@pytest.mark.parametrize("m,topk,e,bs", [(3, 2, 4, 8), (123, 2, 4, 32), (333, 2, 4, 64)])
+def test_moe_gemm_fp4_experts(ops, dev, kind, dtype, m, topk, e, bs):
+    """Per-expert weights, scale bytes and (NVFP4) global scales through moe_wna16_marlin_gemm."""
+    from oracle import moe_ref as mr
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    k, n = 256, 192
+    experts = [make(kind, k, n, dtype, dev, 40 + i) for i in range(e)]
+    mq, ms = torch.stack([x[2] for x in experts]), torch.stack([x[3] for x in experts])
+    gs = torch.cat([x[4] for x in experts]) if kind == "nvfp4" else None
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).to(dtype)
+    g = torch.Generator().manual_seed(6)
+    ids = torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+    tw = torch.rand(m, topk, generator=g)
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e)
+    ws = marlin_make_workspace_new(dev, 4)
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), None, mq, None, ms, gs, None, None, None, ws, s, x, t, tw.to(dev), moe_block_size=bs, top_k=topk,
+        mul_topk_weights=True, is_ep=False, b_q_type=scalar_types.float4_e2m1f, size_m=m, size_n=n, size_k=k,
+        is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
+    ref = mr.moe_gemm_ref(a, torch.stack([x[0] for x in experts]), s.cpu(), x.cpu(), t.cpu(), tw, bs, topk, True, m)
+    mtr = gr.error_metrics(out, ref)
+    assert mtr["max_rel"] <= TOL[dtype] and mtr["mean_rel"] < 0.04, mtr
+    assert int(ws.abs().sum()) == 0

@@ -311,11 +311,26 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
     _check(b_q_weight.size(2) % 16 == 0 and size_n == b_q_weight.size(2) // 16 * pf,
            f"Shape mismatch: b_q_weight.size(2) = {b_q_weight.size(2)}, size_n = {size_n}, pack_factor = {pf}")
     _check(b_scales.is_cuda and b_scales.is_contiguous() and b_scales.dim() == 3, "b_scales rank is not 3")
-    _check(b_scales.size(0) == num_experts and b_scales.size(2) == size_n and b_scales.dtype == a.dtype,
+    _check(b_scales.size(0) == num_experts and b_scales.size(2) == size_n,
            f"b_scales dim 2 = {b_scales.size(2)} is not size_n = {size_n}")
-    _check(not is_zp_float, "float zero points (HQQ) are not implemented by the gfx950 W4A16 library")
-    _check(_opt(global_scale) is None, "global_scale can only be used for nvfp4 format.")
+    _check(not is_zp_float, "float zero points (HQQ) are not implemented for the MoE op by the gfx950 W4A16 library")
     num_groups = b_scales.size(1)
+    gscale = _opt(global_scale)
+    if int(b_q_type_id) == scalar_types.float4_e2m1f.id:
+        group_size = size_k // num_groups if num_groups > 0 and size_k % num_groups == 0 else 0
+        _check(group_size in (16, 32),
+               "float4_e2m1f only supports group_size == 16 (NVFP4) and group_size == 32 (MXFP4)")
+        want = torch.float8_e4m3fn if group_size == 16 else torch.float8_e8m0fnu
+        _check(b_scales.dtype == want, f"b_scales must be {want} for float4_e2m1f with group_size = {group_size}")
+        if group_size == 16:
+            _check(gscale is not None, "the global_scale parameter must be passed for nvfp4 format.")
+            _check(gscale.is_cuda and gscale.is_contiguous() and gscale.numel() == num_experts and
+                   gscale.dtype == a.dtype, "global_scale must hold one element of the activation type per expert")
+        else:
+            _check(gscale is None, "global_scale can only be used for nvfp4 format.")
+    else:
+        _check(b_scales.dtype == a.dtype, "scalar type of a and b_scales must match")
+        _check(gscale is None, "global_scale can only be used for nvfp4 format.")
     g_idx, perm = _opt(g_idx_or_none), _opt(perm_or_none)
     _check((g_idx is None) == (perm is None), "g_idx and perm must both be given or both be empty")
     for name, t in (("g_idx", g_idx), ("perm", perm)):
@@ -367,6 +382,7 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
     args.moe_block_size = moe_block_size
     args.top_k = top_k
     args.num_experts = num_experts
+    args.global_scale = None if gscale is None else gscale.data_ptr()
     _run_gemm(args, a.device)
     return c
 

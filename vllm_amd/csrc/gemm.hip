@@ -39,8 +39,6 @@ static int validate(const w4a16_gemm_args* a) {
                     a->wtype == W4A16_WTYPE_FE2M1,
                 "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False");
   if (a->wtype == W4A16_WTYPE_FE2M1) {
-    if (a->flags & W4A16_F_MOE)
-      return fail(W4A16_ENOTIMPL, "float4_e2m1f weights are not implemented for the MoE op in this build");
     const int64_t gs = a->num_groups > 0 && a->size_k % a->num_groups == 0 ? a->size_k / a->num_groups : 0;
     W4A16_CHECK(gs == 16 || gs == 32, "float4_e2m1f only supports group_size == 16 (NVFP4) and group_size == 32 (MXFP4)");
     W4A16_CHECK(a->g_idx == nullptr, "Unsupported shapes: act-order with float4_e2m1f weights");

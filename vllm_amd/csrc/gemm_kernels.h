@@ -16,7 +16,7 @@ struct KParams {
   const int32_t* gidx;
   const int32_t* perm;
   const void* bias;
-  const void* gscale;  // NVFP4 global scale (one element of the activation type), else null
+  const void* gscale;  // NVFP4 global scale (one element of the activation type per expert), else null
   float* ctmp;
   int32_t* locks;
   int lock_stride;
@@ -139,7 +139,8 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.mul_topk = moe && (a->flags & W4A16_F_MUL_TOPK_WEIGHTS);
   p.n_sorted = moe ? (int)a->n_sorted : 0;
   p.b_estride = (a->size_k / 16) * ((a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) ? 4 : 2) * a->size_n;
-  p.s_estride = a->num_groups * a->size_n;
+  // scale elements are addressed as 16-bit words; fp4 scales are one byte each
+  p.s_estride = a->num_groups * a->size_n / (a->wtype == W4A16_WTYPE_FE2M1 ? 2 : 1);
   p.z_estride = a->num_groups * (a->size_n / 8);
   p.k_estride = a->size_k;
   p.n_estride = a->size_n;

@@ -84,12 +84,14 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const int32_t* gidx = p.gidx;
   const int32_t* perm = p.perm;
   const uint16_t* bias = (const uint16_t*)p.bias;
+  const uint16_t* gscale = (const uint16_t*)p.gscale;
   if (p.moe) {
     if (mt * p.moe_bs >= *p.ntpp) return;
     const int e = p.expert_ids[mt];
     if (e < 0) return;
     Bq += e * p.b_estride;
     Sc += e * p.s_estride;
+    if (FP4 == 1) gscale += e;
     if (ZP) Zp += e * p.z_estride;
     if (gidx) gidx += e * p.k_estride;
     if (PERM) perm += e * p.k_estride;
@@ -450,7 +452,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     }
     if constexpr (FP4 == 1) {
       // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
-      const uint16_t gv = *(const uint16_t*)p.gscale;
+      const uint16_t gv = *gscale;
       const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] *= gs;

@@ -82,7 +82,7 @@ def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, ga
         assert output is None, "Conflicting request"
     quant_type = ScalarType.from_id(quant_type_id)
     assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
-                          scalar_types.float8_e4m3fn), \
+                          scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f), \
         f"unsupported MoE weight type {quant_type}"
     num_bits = quant_type.size_bits
     M, K = hidden_states.size()
@@ -141,7 +141,7 @@ def batched_fused_marlin_moe(hidden_states, expert_num_tokens, w1, w2, bias1, bi
         assert output is None, "Conflicting request."
     quant_type = ScalarType.from_id(quant_type_id)
     assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
-                          scalar_types.float8_e4m3fn), \
+                          scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f), \
         f"unsupported MoE weight type {quant_type}"
     num_bits = quant_type.size_bits
     B, batch_tokens_max, K = hidden_states.size()
