@@ -30,8 +30,8 @@ GROUP = 128
 # HBM bytes per launch of the headline step's GEMM kernel (average of the four launches at M=16), from two
 # `rocprofv3 --pmc` runs of `bench.py --pmc-probe` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same
 # counter reads for the 256 MiB device copy in that run (FETCH_SIZE reads 0.5 per KiB copied, WRITE_SIZE 1.0):
-# read + written KiB: qkv 14629 + 969, o 10648 + 1162, gate_up 60436 + 896, down 34377 + 1162.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = (14629 + 969 + 10648 + 1162 + 60436 + 896 + 34377 + 1162) * 1024 / 4
+# read + written KiB: qkv 14647 + 966, o 10657 + 1160, gate_up 60419 + 896, down 34400 + 1160.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = (14647 + 966 + 10657 + 1160 + 60419 + 896 + 34400 + 1160) * 1024 / 4
 
 
 def algorithmic_bytes(m, k, n, zp=False, act_order=False):
