@@ -90,10 +90,78 @@ def moe_align_cases():
     np.savez_compressed(os.path.join(HERE, "moe_align.npz"), **out)
 
 
+def _regroup_fp4_scales(t):
+    """Regrouping of a Marlin-permuted [G, N] scale matrix for fp4 weights (row pairs interleaved per 8-column chunk,
+    the middle two of every four swapped), the layout the op receives."""
+    g, n = t.shape
+    t = t.view(g // 2, 2, -1, 8).permute(0, 2, 1, 3).reshape(g, n)
+    return t.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(g, n)
+
+
+def other_type_cases():
+    """uint8b128, float zero points (HQQ), float8_e4m3fn and float4_e2m1f (NVFP4, MXFP4): operands as the dense op
+    receives them, the oracle's dequantised weights and its fp32 result."""
+    out = {}
+    g = torch.Generator().manual_seed(14)
+    m, k, n = 5, 256, 64
+    e = torch.empty(0, dtype=torch.int32)
+
+    def put(name, a, mq, scales, w_ref, **extra):
+        out[f"{name}.a"] = bits16(a)
+        out[f"{name}.b_q_weight"] = mq.numpy()
+        out[f"{name}.b_scales"] = scales
+        out[f"{name}.w_ref"] = bits16(w_ref)
+        out[f"{name}.c_ref"] = gr.gemm_ref(a, w_ref).numpy()
+        for key, v in extra.items():
+            out[f"{name}.{key}"] = v
+
+    # uint8b128, group 128, bf16
+    w = (torch.randn(k, n, generator=g) * 0.05).bfloat16()
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w_ref, q, s, _ = qu.quantize_weights(w, st.uint8b128, 128)
+    put("u8b128_bf16_g128", a, ml.gptq_marlin_repack(qu.pack_rows(q, 8), None, k, n, 8),
+        bits16(ml.marlin_permute_scales(s, k, n, 128)), w_ref)
+
+    # HQQ: uint4, fp16 scales and fp16 zero points, group 64
+    q = torch.randint(0, 10, (k, n), generator=g, dtype=torch.int32)
+    s = torch.randn(k // 64, n, generator=g).half()
+    z = torch.randn(k // 64, n, generator=g).half()
+    a = torch.randn(m, k, generator=g).half()
+    mq = ml.gptq_marlin_repack(qu.gptq_pack(q), None, k, n)
+    ms, mz = ml.marlin_permute_scales(s, k, n, 64), ml.marlin_permute_scales(z, k, n, 64)
+    put("hqq_f16_g64", a, mq, bits16(ms), gr.dequant_marlin_float_zp(mq, ms, mz, k, n), b_zeros_f16=bits16(mz))
+
+    # float8_e4m3fn, channel-wise scales, fp16 (scales carry the exponent offset 2^8)
+    w = torch.randn(k, n, generator=g).half()
+    a = torch.randn(m, k, generator=g).half()
+    w_ref, codes, s = qu.quantize_fp8(w, -1)
+    ms = (ml.marlin_permute_scales(s, k, n, k).double() * gr.fp8_scale_offset(torch.float16)).half()
+    put("fp8_f16_chan", a, ml.marlin_weights_closed_form8(codes.to(torch.int32)), bits16(ms), w_ref)
+
+    # float4_e2m1f, NVFP4 (fp16) and MXFP4 (bf16)
+    codes = torch.randint(0, 16, (k, n), generator=g, dtype=torch.int32)
+    mq = ml.gptq_marlin_repack(qu.gptq_pack(codes), None, k, n)
+    a = torch.randn(m, k, generator=g).half()
+    s = (torch.rand(k // 16, n, generator=g) * 3 + 0.02).to(torch.float8_e4m3fn).half()
+    ms = _regroup_fp4_scales(ml.marlin_permute_scales(s, k, n, 16))
+    byts = ((ms * 128).view(torch.int16) << 1).view(torch.uint8)[:, 1::2].contiguous()
+    gs = torch.tensor([0.0371], dtype=torch.float16)
+    gs_proc = (gs.double() * 2.0 ** 7).half()
+    put("nvfp4_f16", a, mq, byts.numpy(), gr.dequant_marlin_fp4(mq, byts, gs_proc, k, n, torch.float16),
+        global_scale=bits16(gs_proc))
+    a = torch.randn(m, k, generator=g).bfloat16()
+    sb = torch.randint(110, 125, (k // 32, n), generator=g, dtype=torch.uint8)
+    ms = _regroup_fp4_scales(ml.marlin_permute_scales(sb.view(torch.float8_e8m0fnu).to(torch.bfloat16), k, n, 32))
+    byts = ms.to(torch.float8_e8m0fnu).view(torch.uint8).contiguous()
+    put("mxfp4_bf16", a, mq, byts.numpy(), gr.dequant_marlin_fp4(mq, byts, None, k, n, torch.bfloat16))
+    np.savez_compressed(os.path.join(HERE, "other_types.npz"), **out)
+
+
 if __name__ == "__main__":
     repack_cases()
     gemm_cases()
     moe_align_cases()
+    other_type_cases()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

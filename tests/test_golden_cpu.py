@@ -66,3 +66,33 @@ def test_moe_align_fixtures():
         assert np.array_equal(s.numpy(), z[f"{c}.sorted_ids"])
         assert np.array_equal(x.numpy(), z[f"{c}.expert_ids"])
         assert np.array_equal(t.numpy(), z[f"{c}.total"])
+
+
+def _other_type_w(z, c):
+    """The oracle's dequantised weights for one case of other_types.npz, from the stored operands."""
+    dtype = torch.bfloat16 if "bf16" in c else torch.float16
+    mq = torch.from_numpy(z[f"{c}.b_q_weight"].copy())
+    k = mq.shape[0] * 16
+    if c.startswith("u8b128"):
+        n = mq.shape[1] // 4
+        return gr.dequant_marlin(mq, from_bits(z[f"{c}.b_scales"], dtype), None, None, k, n, True, dtype, num_bits=8)
+    if c.startswith("fp8"):
+        return gr.dequant_marlin_fp8(mq, from_bits(z[f"{c}.b_scales"], dtype), k, mq.shape[1] // 4, dtype)
+    n = mq.shape[1] // 2
+    if c.startswith("hqq"):
+        return gr.dequant_marlin_float_zp(mq, from_bits(z[f"{c}.b_scales"], dtype),
+                                          from_bits(z[f"{c}.b_zeros_f16"], dtype), k, n)
+    byts = torch.from_numpy(z[f"{c}.b_scales"].copy())
+    gs = from_bits(z[f"{c}.global_scale"], dtype) if f"{c}.global_scale" in z.files else None
+    return gr.dequant_marlin_fp4(mq, byts, gs, k, n, dtype)
+
+
+def test_other_type_fixtures():
+    z = load("other_types.npz")
+    assert cases(z) == ["fp8_f16_chan", "hqq_f16_g64", "mxfp4_bf16", "nvfp4_f16", "u8b128_bf16_g128"]
+    for c in cases(z):
+        dtype = torch.bfloat16 if "bf16" in c else torch.float16
+        w = _other_type_w(z, c)
+        assert torch.equal(w, from_bits(z[f"{c}.w_ref"], dtype)), c
+        a = from_bits(z[f"{c}.a"], dtype)
+        assert np.array_equal(gr.gemm_ref(a, w).numpy(), z[f"{c}.c_ref"]), c

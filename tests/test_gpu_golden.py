@@ -72,3 +72,45 @@ def test_moe_align_fixtures_exact(dev):
         assert np.array_equal(t.cpu().numpy(), z[f"{c}.total"]), c
         assert np.array_equal(s.cpu().numpy(), z[f"{c}.sorted_ids"]), c
         assert np.array_equal(x.cpu().numpy(), z[f"{c}.expert_ids"]), c
+
+
+def test_other_type_fixtures(dev):
+    """uint8b128, float zero points, float8_e4m3fn and float4_e2m1f operands of tests/golden/other_types.npz."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.scalar_type import scalar_types
+    z = load("other_types.npz")
+    ws = marlin_make_workspace_new(dev)
+    wtypes = {"u8b128": scalar_types.uint8b128, "hqq": scalar_types.uint4, "fp8": scalar_types.float8_e4m3fn,
+              "nvfp4": scalar_types.float4_e2m1f, "mxfp4": scalar_types.float4_e2m1f}
+    for c in cases(z):
+        kind = c.split("_")[0]
+        dtype = torch.bfloat16 if "bf16" in c else torch.float16
+        bits = lambda key: torch.from_numpy(z[f"{c}.{key}"].copy()).view(dtype).to(dev)
+        a = bits("a")
+        mq = torch.from_numpy(z[f"{c}.b_q_weight"].copy()).to(dev)
+        k = a.shape[1]
+        n = mq.shape[1] // (4 if kind in ("u8b128", "fp8") else 2)
+        zeros, gs, zp_float = None, None, False
+        if kind in ("nvfp4", "mxfp4"):
+            raw = torch.from_numpy(z[f"{c}.b_scales"].copy()).to(dev)
+            scales = raw.view(torch.float8_e4m3fn if kind == "nvfp4" else torch.float8_e8m0fnu)
+            gs = bits("global_scale") if kind == "nvfp4" else None
+        else:
+            scales = bits("b_scales")
+        if kind == "hqq":
+            zeros, zp_float = bits("b_zeros_f16"), True
+
+        def run(x):
+            return ops.gptq_marlin_gemm(x, None, mq, None, scales, gs, zeros, None, None, ws, wtypes[kind], x.shape[0], n, k,
+                                        True, False, True, zp_float)
+        ref = torch.from_numpy(z[f"{c}.c_ref"])
+        d = (run(a).float().cpu() - ref).abs()
+        assert float(d.max() / ref.abs().max()) <= (4e-2 if dtype == torch.bfloat16 else 2e-2), c
+        assert float(d.mean() / ref.abs().mean()) < 0.04, c
+        rows = torch.tensor([0, 1, 17, k // 2 + 3, k - 1])
+        onehot = torch.zeros(len(rows), k, dtype=dtype)
+        onehot[torch.arange(len(rows)), rows] = 1
+        w_ref = torch.from_numpy(z[f"{c}.w_ref"].copy()).view(dtype)
+        assert torch.equal(run(onehot.to(dev)).cpu(), w_ref[rows]), c
+        assert int(ws.abs().sum()) == 0
