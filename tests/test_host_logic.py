@@ -126,3 +126,15 @@ def test_kernel_selection_rejects_unsupported_configs():
     ok, why = MarlinLinearKernel.can_implement(c)
     if not torch.cuda.is_available():
         assert not ok and "ROCm device" in why
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message instead of a JSON line."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
