@@ -146,7 +146,20 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool perm_in_kernel = act_order && moe;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
-  if (!moe && !general_only && pow2_group && a->size_m >= 128 && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  // ... unless the same problem cut into 64-row tiles finishes sooner.  In units of one 128 x 512 tile's time (measured):
+  // a round of 128-row tiles costs 1 (0.6 when its trailing strips are handed to the 64-row kernel); 64-row tiles cost
+  // 0.75 with one workgroup per compute unit and 1.15 per pair with two.  (2048 x 4096: 128 tiles of 128 rows leave
+  // half the compute units idle, 256 tiles of 64 rows do not: 99 -> 75 us at K = 4096.)
+  bool prefer_mid = false;
+  if (fat_tiles >= cus / 2 && forced_kind < 0) {
+    const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
+    const bool handoff = fat_tiles >= cus && tail > 0 && tail * 2 <= cus && tail % mt128 == 0;
+    const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.6 : 1.0);
+    const int64_t mid_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 512), rem = mid_tiles % (2 * cus);
+    const double mid_units = 1.15 * (double)(mid_tiles / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.75 : 1.15);
+    prefer_mid = mid_units < 0.95 * fat_units;
+  }
+  if (!moe && !general_only && pow2_group && a->size_m >= 128 && !prefer_mid && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
