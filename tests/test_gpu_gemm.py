@@ -264,17 +264,21 @@ def test_reduce_flags_do_not_change_results(ops, dev, workspace):
     check_close(outs[0], a, layer)
 
 
-def test_prefill_tail_strips_go_to_the_64_row_kernel(ops, dev, workspace):
-    """4096 x 6144: 384 tiles of 128 x 512 = one full round of the 256 compute units plus half a round; the last four
-    512-column strips are computed by the 64-row kernel.  Both halves must meet the same bar."""
-    size_m, size_k, size_n = 4096, 256, 6144
+@pytest.mark.parametrize("size_m,handed", [(4096, 4), (3072, 2), (2100, 1)])
+def test_prefill_tail_strips_go_to_the_64_row_kernel(ops, dev, workspace, size_m, handed):
+    """N = 6144 in 128 x 512 tiles on 256 compute units: 4096 rows give one full round plus half a round (four whole
+    strips), 3072 rows one round plus 32 tiles (one strip and a third), 2100 rows 204 tiles (no second round: `handed`
+    strips only if a second round exists).  The handed-over strips are computed by the 64-row kernel; both parts must
+    meet the same bar."""
+    size_k, size_n = 256, 6144
     layer = make_layer(size_k, size_n, 128, torch.bfloat16, has_zp=True, seed=41, rule="minmax", w_std=0.05)
     a = _a(size_m, size_k, torch.bfloat16, dev)
     bias = torch.randn(size_n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
     from vllm_amd.marlin_utils import marlin_permute_bias
     out = run_gemm(ops, layer, a, dev, workspace, bias=marlin_permute_bias(bias.to(dev)))
     ref = gr.gemm_ref(a.cpu(), layer.w_ref, bias)
-    for lo, hi in ((0, 4096), (4096, 6144)):      # prefill-kernel strips, 64-row-kernel strips
+    split = size_n - 512 * handed
+    for lo, hi in ((0, split), (split, size_n)):      # prefill-kernel strips, strips that may be handed over
         m = gr.error_metrics(out[:, lo:hi], ref[:, lo:hi])
         assert m["max_rel"] <= 4e-2 and m["mean_rel"] < 0.04, (lo, hi, m)
 

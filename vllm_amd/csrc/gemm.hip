@@ -153,8 +153,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   bool prefer_mid = false;
   if (fat_tiles >= cus / 2 && forced_kind < 0) {
     const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
-    const bool handoff = fat_tiles >= cus && tail > 0 && tail * 2 <= cus && tail % mt128 == 0;
-    const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.6 : 1.0);
+    const bool handoff = fat_tiles >= cus && tail > 0 && ceil_div(tail, mt128) * ceil_div(a->size_m, 64) <= cus;
+    const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.7 : 1.0);
     const int64_t mid_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 512), rem = mid_tiles % (2 * cus);
     const double mid_units = 1.15 * (double)(mid_tiles / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.75 : 1.15);
     prefer_mid = mid_units < 0.95 * fat_units;
@@ -174,13 +174,14 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = pl.total_ksteps;
     pl.xcd_map = 0;
     pl.ctmp_bytes = 0;
-    // One workgroup fills a compute unit, so tiles run in rounds of `cus`.  When the last round is at most half full
-    // and consists of whole 512-column strips (tiles are ordered M first), those strips go to the 64-row kernel instead:
-    // twice as many, half-size workgroups occupy every compute unit for about two thirds of a round.
+    // One workgroup fills a compute unit, so tiles run in rounds of `cus`.  The strips that reach into a partly filled
+    // last round (tiles are ordered M first) go to the 64-row kernel instead when it can hold them with one workgroup
+    // per compute unit: that takes about 0.75 of a round instead of a whole one.
     {
       const int64_t rounds = tiles / cus, tail = tiles - rounds * cus;
-      if (rounds >= 1 && tail > 0 && tail * 2 <= cus && tail % pl.mtiles == 0 && forced_kind != 2)
-        pl.tail_strips = (int)(tail / pl.mtiles);
+      const int64_t strips = ceil_div(tail, (int64_t)pl.mtiles);
+      if (rounds >= 1 && tail > 0 && strips < pl.ncp && strips * ceil_div(a->size_m, 64) <= cus && forced_kind != 2)
+        pl.tail_strips = (int)strips;
     }
     return 0;
   }
