@@ -138,3 +138,47 @@ def test_moe_gemm_fp4_experts(ops, dev, kind, dtype, m, topk, e, bs):
     mtr = gr.error_metrics(out, ref)
     assert mtr["max_rel"] <= TOL[dtype] and mtr["mean_rel"] < 0.04, mtr
     assert int(ws.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("mxfp4", torch.bfloat16), ("fp8", torch.bfloat16)])
+@pytest.mark.parametrize("m", [1, 33, 200])
+def test_fused_marlin_moe_with_float_weight_types(dev, kind, dtype, m):
+    """fused_marlin_moe end to end (align, GEMM1, SiLU-and-mul, GEMM2, sum) with fp4 / fp8 experts and per-expert
+    global scales, against torch_experts on the oracle's dequantised weights (the reference's gate: atol 5e-2)."""
+    from oracle import marlin_layout as ml
+    from oracle import moe_ref as mr
+    from oracle import quant_utils as qu
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    from vllm_amd.scalar_type import scalar_types
+    e, topk, k, inter = 4, 2, 256, 128
+
+    def experts(size_k, size_n, seed):
+        if kind == "fp8":
+            ws, qs, ss = [], [], []
+            for i in range(e):
+                w = (torch.randn(size_k, size_n, generator=torch.Generator().manual_seed(seed + i)) * 0.1).to(dtype)
+                w_ref, codes, s = qu.quantize_fp8(w, 128)
+                ms = ml.marlin_permute_scales(s, size_k, size_n, 128)
+                ws.append(w_ref)
+                qs.append(ml.marlin_weights_closed_form8(codes.to(torch.int32)))
+                ss.append((ms.double() * gr.fp8_scale_offset(dtype)).to(dtype))
+            return torch.stack(ws), torch.stack(qs).to(dev), torch.stack(ss).to(dev), None
+        made = [make(kind, size_k, size_n, dtype, dev, seed + i) for i in range(e)]
+        gs = torch.cat([x[4] for x in made]) if kind == "nvfp4" else None
+        return torch.stack([x[0] for x in made]), torch.stack([x[2] for x in made]), torch.stack([x[3] for x in made]), gs
+
+    w1, q1, s1, g1 = experts(k, 2 * inter, 300)
+    w2, q2, s2, g2 = experts(inter, k, 400)
+    g = torch.Generator().manual_seed(12)
+    a_scale = 0.1 if kind == "fp8" else 0.01
+    a = (torch.randn(m, k, generator=g) * a_scale).to(dtype)
+    score = torch.randn(m, e, generator=g).to(dtype)
+    tw, ti = torch.topk(torch.softmax(score.float(), dim=-1), topk)
+    wtype = scalar_types.float8_e4m3fn if kind == "fp8" else scalar_types.float4_e2m1f
+    out = fused_marlin_moe(a.to(dev), q1, q2, None, None, s1, s2, score.to(dev), tw.to(dev), ti.to(torch.int32).to(dev),
+                           quant_type_id=wtype.id, global_num_experts=e, global_scale1=g1, global_scale2=g2)
+    ref = mr.torch_experts(a, w1.transpose(1, 2), w2.transpose(1, 2), tw, ti)
+    assert out.shape == (m, k)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=max(5e-2, 2e-2 * float(ref.abs().max())), rtol=0)
+    mtr = gr.error_metrics(out, ref)          # and relative to the result's own size (two GEMMs and a 16-bit intermediate)
+    assert mtr["max_rel"] <= 2 * TOL[dtype] and mtr["mean_rel"] < 0.04, mtr
