@@ -138,3 +138,31 @@ def test_bench_refuses_more_than_one_gpu():
                        timeout=120)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_support_queries_and_layer_checks():
+    import types
+    from vllm_amd import marlin_utils as mu
+    from vllm_amd.scalar_type import scalar_types
+    assert mu.check_marlin_supported(scalar_types.uint4b8, 128) and mu.check_marlin_supported(scalar_types.uint4, 64, True)
+    assert not mu.check_marlin_supported(scalar_types.uint4, 128)              # uint4 needs zero points
+    assert not mu.check_marlin_supported(scalar_types.uint4b8, 100)
+    with pytest.raises(ValueError, match="does not support group_size = 100"):
+        mu.verify_marlin_supported(scalar_types.uint4b8, 100)
+    with pytest.raises(ValueError, match="does not support weight_bits = uint4"):
+        mu.verify_marlin_supported(scalar_types.uint4, 128)
+    layer = types.SimpleNamespace(output_size_per_partition=6144, input_size_per_partition=4096, input_size=4096,
+                                  output_size=6144)
+    assert mu.check_marlin_supports_layer(layer, 128)
+    layer.input_size_per_partition = 4000
+    assert not mu.check_marlin_supports_layer(layer, 128)
+    moe = types.SimpleNamespace(hidden_size=4096, intermediate_size_per_partition=14336,
+                                apply_router_weight_on_input=False, activation="silu")
+    assert mu.check_moe_marlin_supports_layer(moe, 128)
+    moe.activation = "gelu"
+    assert not mu.check_moe_marlin_supports_layer(moe, 128)
+    moe.activation, moe.intermediate_size_per_partition = "silu", 14336 + 32
+    assert not mu.check_moe_marlin_supports_layer(moe, 128)
+    import torch
+    assert mu.marlin_moe_intermediate_size(torch.empty(8, 256, 57344), torch.empty(8, 896, 8192)) == 14336
+    assert mu.marlin_make_workspace(4096, torch.device("cpu")).shape == (1024,)

@@ -6,7 +6,7 @@ from collections.abc import Callable
 import torch
 
 from . import _custom_ops as ops
-from .marlin_utils import marlin_make_workspace_new
+from .marlin_utils import marlin_make_workspace_new, marlin_moe_intermediate_size
 from .moe_align_block_size import batched_moe_align_block_size, moe_align_block_size
 from .scalar_type import ScalarType, scalar_types
 
@@ -16,11 +16,6 @@ def default_activation_func(activation: str, output: torch.Tensor, input: torch.
         ops.silu_and_mul(output, input)
     else:
         raise ValueError(f"Unsupported activation: {activation}. Only silu is implemented.")
-
-
-def marlin_moe_intermediate_size(w1_packed: torch.Tensor, w2_packed: torch.Tensor) -> int:
-    """w2 is [E, N/16, K * bits/2]: rows of 16-row k-tiles of the intermediate size N."""
-    return w2_packed.size(1) * 16
 
 
 def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk: int,

@@ -59,6 +59,56 @@ def verify_marlin_supports_shape(output_size_per_partition: int, input_size_per_
                          "--quantization gptq.")
 
 
+def _check_marlin_supported(quant_type: ScalarType, group_size: int | None, has_zp: bool,
+                            device_capability: int | None = None) -> tuple[bool, str | None]:
+    """Type and group-size gate with the reference's messages (marlin_utils.py:72-104)."""
+    supported_types = query_marlin_supported_quant_types(has_zp, True, device_capability)
+    if quant_type not in supported_types:
+        return False, (f"Marlin does not support weight_bits = {quant_type}. Only types = "
+                       f"{[str(t) for t in supported_types]} are supported (for group_size = {group_size}, "
+                       f"device_capability = {device_capability}, zp = {has_zp}).")
+    if group_size is None or group_size not in MARLIN_SUPPORTED_GROUP_SIZES:
+        return False, (f"Marlin does not support group_size = {group_size}. Only group_sizes = "
+                       f"{MARLIN_SUPPORTED_GROUP_SIZES} are supported.")
+    return True, None
+
+
+def check_marlin_supported(quant_type: ScalarType, group_size: int, has_zp: bool = False,
+                           device_capability: int | None = None) -> bool:
+    return _check_marlin_supported(quant_type, group_size, has_zp, device_capability)[0]
+
+
+def verify_marlin_supported(quant_type: ScalarType, group_size: int, has_zp: bool = False) -> None:
+    ok, msg = _check_marlin_supported(quant_type, group_size, has_zp)
+    if not ok:
+        raise ValueError(msg)
+
+
+def check_marlin_supports_layer(layer, group_size: int) -> bool:
+    """marlin_utils.py:176-189: the layer's partition sizes (or its full sizes) against the shape gates."""
+    out_size = getattr(layer, "output_size_per_partition", None) or layer.output_size
+    in_size = getattr(layer, "input_size_per_partition", None) or layer.input_size
+    return check_marlin_supports_shape(out_size, in_size, layer.input_size, group_size)[0]
+
+
+def check_moe_marlin_supports_layer(layer, group_size: int) -> bool:
+    """marlin_utils.py:192-213: hidden % 128, intermediate % max(64, group), SiLU, router weight on the output."""
+    shape_ok = layer.hidden_size % 128 == 0 and layer.intermediate_size_per_partition % max(64, group_size) == 0
+    return (shape_ok and group_size in (-1, 32, 64, 128) and not layer.apply_router_weight_on_input and
+            layer.activation == "silu")
+
+
+def marlin_moe_intermediate_size(w1_packed: torch.Tensor, w2_packed: torch.Tensor) -> int:
+    """w2 is [E, N/16, ...]: rows are 16-row k-tiles of the intermediate size N (marlin_utils.py:216-222)."""
+    return w2_packed.size(1) * GPTQ_MARLIN_TILE
+
+
+def marlin_make_workspace(output_size_per_partition: int, device: torch.device) -> torch.Tensor:
+    """The older sizing rule, (N / 64) * 16 zeroed ints (marlin_utils.py:225-234); any all-zero int32 tensor works."""
+    size = (output_size_per_partition // GPTQ_MARLIN_MIN_THREAD_N) * GPTQ_MARLIN_MAX_PARALLEL
+    return torch.zeros(size, dtype=torch.int, device=device, requires_grad=False)
+
+
 def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1) -> torch.Tensor:
     """int32 zeros, four counters per compute unit (x max_blocks_per_sm); the reference's function
     (marlin_utils.py:237-245) allocates one per SM, which the GEMM also accepts: the extra length only lets it place
@@ -181,4 +231,20 @@ def apply_awq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_sc
                                   size_n=output_size_per_partition, size_k=input_size_per_partition,
                                   use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,
                                   is_zp_float=False)
+    return output.reshape(out_shape)
+
+
+def apply_rtn_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                            workspace: torch.Tensor, quant_type: ScalarType, output_size_per_partition: int,
+                            input_size_per_partition: int, bias: torch.Tensor | None = None,
+                            use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    """Round-to-nearest checkpoints: symmetric weights, no zero points, no act-order (marlin_utils.py:533-577)."""
+    reshaped_x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (output_size_per_partition,)
+    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
+                                                  reshaped_x.size(1), input.device, input.dtype)
+    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, None, None, None, workspace,
+                                  quant_type, size_m=reshaped_x.shape[0], size_n=output_size_per_partition,
+                                  size_k=input_size_per_partition, use_atomic_add=use_atomic_add,
+                                  use_fp32_reduce=use_fp32_reduce, is_zp_float=False)
     return output.reshape(out_shape)
