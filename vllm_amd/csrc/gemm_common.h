@@ -317,6 +317,47 @@ __device__ __forceinline__ void dequant_pair_fp4(uint32_t xa, uint32_t xb, float
   o0 = u32x4{p0, p1, p2, p3};
   o1 = u32x4{q0, q1, q2, q3};
 }
+// Direct fp4 -> 16-bit conversion: v_cvt_scalef32_pk_{f16,bf16}_fp4 turns one byte (the codes of K rows k0 and
+// k0+8 of one column) into a packed 16-bit pair, times 2^(exponent of `scale` - 127).  The B operand of a column half
+// is then in the K order (k0, k0+8, k0+1, k0+9, 16+k0, 24+k0, 17+k0, 25+k0) instead of (k0, k0+1, k0+8, k0+9, ...):
+// the A operand is reordered to match (a_frag_fp4_order), which costs 4 v_perm_b32 per m-block and k-step instead of
+// two multiplies and a pack per weight pair.
+template <int DT, int BYTE>
+__device__ __forceinline__ uint32_t cvt_fp4x2(uint32_t x, float scale) {
+  if constexpr (DT == DT_F16) {
+    return as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(x, scale, BYTE));
+  } else {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    const bf2 r = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x, scale, BYTE);
+    return __builtin_bit_cast(uint32_t, r);
+  }
+}
+__device__ __forceinline__ u32x4 a_frag_fp4_order(u32x4 a) {
+  return u32x4{__builtin_amdgcn_perm(a[1], a[0], 0x05040100u), __builtin_amdgcn_perm(a[1], a[0], 0x07060302u),
+               __builtin_amdgcn_perm(a[3], a[2], 0x05040100u), __builtin_amdgcn_perm(a[3], a[2], 0x07060302u)};
+}
+// MXFP4: the E8M0 group scale is the conversion's scale operand (exact: a power of two).  s0 / s1: scale of column
+// half 0 / 1 as fp32 (only its exponent is used).
+template <int DT>
+__device__ __forceinline__ void dequant_pair_mxfp4_direct(uint32_t xa, uint32_t xb, float s0, float s1, u32x4& o0,
+                                                          u32x4& o1) {
+  o0 = u32x4{cvt_fp4x2<DT, 0>(xa, s0), cvt_fp4x2<DT, 2>(xa, s0), cvt_fp4x2<DT, 0>(xb, s0), cvt_fp4x2<DT, 2>(xb, s0)};
+  o1 = u32x4{cvt_fp4x2<DT, 1>(xa, s1), cvt_fp4x2<DT, 3>(xa, s1), cvt_fp4x2<DT, 1>(xb, s1), cvt_fp4x2<DT, 3>(xb, s1)};
+}
+// NVFP4, fp16: the scale byte b stands for the half (b << 7) = s * 2^7.  The codes are converted times 2^-7 (exact,
+// >= 2^-8) and multiplied by that half with one packed multiply: value * s rounded once, as the fp32 route gives.
+// ba / bb: scale bytes of k-tile a / b, column half 0 in bits 0..7, half 1 in bits 16..23.
+__device__ __forceinline__ void dequant_pair_nvfp4_f16_direct(uint32_t xa, uint32_t xb, uint32_t ba, uint32_t bb,
+                                                              u32x4& o0, u32x4& o1) {
+  const float pre = 0x1.0p-7f;
+  auto h2 = [](uint32_t byte) { return as_h2(byte * 0x00800080u); };  // (b << 7) in both halves
+  const f16x2 sa0 = h2(ba & 0xffu), sa1 = h2(ba >> 16), sb0 = h2(bb & 0xffu), sb1 = h2(bb >> 16);
+  auto m = [](uint32_t v, f16x2 sc) { return as_u32(as_h2(v) * sc); };
+  o0 = u32x4{m(cvt_fp4x2<DT_F16, 0>(xa, pre), sa0), m(cvt_fp4x2<DT_F16, 2>(xa, pre), sa0),
+             m(cvt_fp4x2<DT_F16, 0>(xb, pre), sb0), m(cvt_fp4x2<DT_F16, 2>(xb, pre), sb0)};
+  o1 = u32x4{m(cvt_fp4x2<DT_F16, 1>(xa, pre), sa1), m(cvt_fp4x2<DT_F16, 3>(xa, pre), sa1),
+             m(cvt_fp4x2<DT_F16, 1>(xb, pre), sb1), m(cvt_fp4x2<DT_F16, 3>(xb, pre), sb1)};
+}
 // Scale bytes of Marlin word w in a lane's 16-byte fp4 scale record: 8 bytes per k-tile (NVFP4) or k-step (MXFP4),
 // stored in the order (e0, e2, e1, e3, e4, e6, e5, e7) with e = 2w + half (marlin_utils_fp4.py:44-47, 68-71).
 // half_rec: the 8 bytes as two dwords; returns byte of column half 0 in bits 0..7 and of half 1 in bits 16..23.

@@ -55,6 +55,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
   constexpr bool FOLD = (MB == 1) && (GM != GM_GIDX) && (BITS == 4) && !ZPF && FP4 == 0;
   constexpr bool HI_TRICK = FOLD && (DT == DT_F16) && !ZP;
+  // fp4 codes converted straight to the 16-bit type (A reordered to the resulting K order); NVFP4 with bf16 has no
+  // packed multiply for the scale mantissa and stays on the fp32 route
+  constexpr bool FP4_DIRECT = (FP4 == 2) || (FP4 == 1 && DT == DT_F16);
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
   __shared__ int s_last;
@@ -210,7 +213,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   auto dequant_word = [&](const Stage& s, auto w_tag, auto unit_tag, u32x4& o0, u32x4& o1) {
     constexpr int w = decltype(w_tag)::value;
     constexpr bool unit = decltype(unit_tag)::value;
-    if constexpr (FP4 == 1) {
+    if constexpr (FP4 == 1 && FP4_DIRECT) {
+      const uint32_t ba = fp4_scale_bytes(s.sc[0], s.sc[1], w), bb = fp4_scale_bytes(s.sc[2], s.sc[3], w);
+      dequant_pair_nvfp4_f16_direct(s.b0[w], s.b1[w], ba, bb, o0, o1);
+    } else if constexpr (FP4 == 2 && FP4_DIRECT) {
+      const uint32_t bs = s.zq ? fp4_scale_bytes(s.sc[2], s.sc[3], w) : fp4_scale_bytes(s.sc[0], s.sc[1], w);
+      dequant_pair_mxfp4_direct<DT>(s.b0[w], s.b1[w], mxfp4_scale_f32(bs & 0xff), mxfp4_scale_f32(bs >> 16), o0, o1);
+    } else if constexpr (FP4 == 1) {
       const uint32_t ba = fp4_scale_bytes(s.sc[0], s.sc[1], w), bb = fp4_scale_bytes(s.sc[2], s.sc[3], w);
       dequant_pair_fp4<DT>(s.b0[w], s.b1[w], nvfp4_scale_f32(ba & 0xff), nvfp4_scale_f32(ba >> 16),
                            nvfp4_scale_f32(bb & 0xff), nvfp4_scale_f32(bb >> 16), o0, o1);
@@ -292,6 +301,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     for (int mb = 0; mb < MB; ++mb) {
       const uint32_t* q = slab_rd + mb * 16 * A_ROW;
       af[mb] = u32x4{q[0], q[4], q[8], q[12]};
+      if constexpr (FP4_DIRECT) af[mb] = a_frag_fp4_order(af[mb]);
     }
     }
     if constexpr (FOLD) {
