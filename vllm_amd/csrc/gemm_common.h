@@ -19,6 +19,8 @@
 // The accumulator of lane l holds rows 4(l>>4) .. +3 of column label l & 15 — the lane's own
 // columns, so per-column scales / zero-points / bias never cross lanes.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace w4a16 {
@@ -290,6 +292,44 @@ __device__ __forceinline__ void dequant_pair8_fp8(uint32_t xa0, uint32_t xa1, ui
   cvt(xb1, s1, q2, q3);
   o0 = u32x4{p0, p1, p2, p3};
   o1 = u32x4{q0, q1, q2, q3};
+}
+
+// The same weights converted straight to the 16-bit type: v_cvt_scalef32_pk_{f16,bf16}_fp8 turns the two low (or high)
+// bytes of a word, K rows (k0, k0+8) or (k0+1, k0+9), into a packed pair times 2^(exponent of scale - 127); the B
+// operand is then in the K order (k0, k0+8, k0+1, k0+9, ...) and A is reordered to match (a_frag_fp4_order).
+// fp16: codes * 2^-8 (exact, takes the exponent offset out of the stored scale), then one packed multiply by the
+// stored scale: x * s rounded once, as above.  Without a per-element scale (channel-wise) the conversion alone is exact
+// in either type.
+template <int DT, bool UNIT_SCALE>
+__device__ __forceinline__ void dequant_pair8_fp8_direct(uint32_t xa0, uint32_t xa1, uint32_t xb0, uint32_t xb1,
+                                                         uint32_t s_pair, u32x4& o0, u32x4& o1) {
+  static_assert(DT == DT_F16 || UNIT_SCALE, "bf16 has no packed multiply");
+  const float pre = UNIT_SCALE ? 1.0f : 0x1.0p-8f;
+  auto cvt = [&](uint32_t x, auto hi_tag) {
+    constexpr bool hi = decltype(hi_tag)::value;
+    if constexpr (DT == DT_F16) {
+      return as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, pre, hi));
+    } else {
+      typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+      const bf2 r = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x, pre, hi);
+      return __builtin_bit_cast(uint32_t, r);
+    }
+  };
+  using T = std::integral_constant<bool, true>;
+  using F = std::integral_constant<bool, false>;
+  u32x4 r0 = {cvt(xa0, F{}), cvt(xa0, T{}), cvt(xb0, F{}), cvt(xb0, T{})};
+  u32x4 r1 = {cvt(xa1, F{}), cvt(xa1, T{}), cvt(xb1, F{}), cvt(xb1, T{})};
+  if constexpr (!UNIT_SCALE) {
+    const f16x2 s = as_h2(s_pair);
+    const f16x2 s0 = {s.x, s.x}, s1 = {s.y, s.y};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      r0[i] = as_u32(as_h2(r0[i]) * s0);
+      r1[i] = as_u32(as_h2(r1[i]) * s1);
+    }
+  }
+  o0 = r0;
+  o1 = r1;
 }
 
 // fp4 (float4_e2m1f) weights in the 4-bit Marlin layout.  A byte of a Marlin word holds the codes of K rows (k0, k0+8)

@@ -58,6 +58,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   // fp4 codes converted straight to the 16-bit type (A reordered to the resulting K order); NVFP4 with bf16 has no
   // packed multiply for the scale mantissa and stays on the fp32 route
   constexpr bool FP4_DIRECT = (FP4 == 2) || (FP4 == 1 && DT == DT_F16);
+  // fp8 likewise, where the scale can follow as a packed fp16 multiply or is applied to the accumulator (channel-wise)
+  constexpr bool FP8_DIRECT = FP8 && (DT == DT_F16 || GM == GM_CHANNEL);
+  constexpr bool A_PAIR_ORDER = FP4_DIRECT || FP8_DIRECT;  // A fragments in the K order (k0, k0+8, k0+1, k0+9, ...)
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
   __shared__ int s_last;
@@ -241,7 +244,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     } else {
       const u32x4& la = (w < 2) ? s.b0 : s.b0h;
       const u32x4& lb = (w < 2) ? s.b1 : s.b1h;
-      if constexpr (FP8)
+      if constexpr (FP8_DIRECT)
+        dequant_pair8_fp8_direct<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
+                                           unit ? 0u : s.sc[w], o0, o1);
+      else if constexpr (FP8)
         dequant_pair8_fp8<DT, unit>(la[2 * (w & 1)], la[2 * (w & 1) + 1], lb[2 * (w & 1)], lb[2 * (w & 1) + 1],
                                     unit ? 0u : s.sc[w], o0, o1);
       else
@@ -301,7 +307,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     for (int mb = 0; mb < MB; ++mb) {
       const uint32_t* q = slab_rd + mb * 16 * A_ROW;
       af[mb] = u32x4{q[0], q[4], q[8], q[12]};
-      if constexpr (FP4_DIRECT) af[mb] = a_frag_fp4_order(af[mb]);
+      if constexpr (A_PAIR_ORDER) af[mb] = a_frag_fp4_order(af[mb]);
     }
     }
     if constexpr (FOLD) {
