@@ -60,6 +60,9 @@ def load() -> ctypes.CDLL:
             raise ImportError(
                 f"{LIB_PATH} not found: build it with `python -m vllm_amd.build` (hipcc, gfx950). "
                 "There is no fallback implementation.")
+        # torch first: it brings its own HIP runtime, and this library must bind to that same instance (loaded the
+        # other way round the process holds two runtimes, and launches here fail with "no ROCm-capable device")
+        import torch  # noqa: F401
         lib = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in EXPORTS.items():
             fn = getattr(lib, name)
