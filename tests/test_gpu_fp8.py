@@ -85,6 +85,26 @@ def test_reference_grid(ops, dev, workspace, dtype, group, n_chunk, mnk):
     assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 128])
+def test_prefill_tiles(ops, dev, workspace, dtype, group):
+    """Enough 128-row tiles for the prefill kernel, with a partial row tile and a partial 512-column strip: random
+    activations against the oracle, one-hot rows bit-exact."""
+    size_m, size_k, size_n = 1100, 512, 8256
+    print(f"fp8 prefill dtype={dtype} g={group}", flush=True)
+    w_ref, _, mq, ms = make_fp8(size_k, size_n, group, dtype, 17)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).to(dtype)
+    out = run(ops, a.to(dev), mq, ms, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w_ref))
+    assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w_ref[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_host_helpers_match_the_oracle(ops, dev, workspace):
     """marlin_quant_fp8_torch (repack op + scale permutation + exponent offset) against the oracle's tensors, and
     apply_fp8_marlin_linear with a bias."""

@@ -59,6 +59,25 @@ def test_gemm_w8(ops, dev, workspace, dtype, m, group, act_order, k_full):
     assert int(workspace.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group,act_order", [(-1, False), (128, False), (64, True)])
+def test_prefill_tiles_w8(ops, dev, workspace, dtype, group, act_order):
+    """Enough 128-row tiles for the prefill kernel (M = 1100 leaves a partial row tile, N = 8256 a partial 512-column
+    strip): random activations against the oracle, and one-hot rows bit-exact on the same launch shape."""
+    m, k, n = 1100, 512, 8256
+    print(f"w8 prefill dtype={dtype} g={group} act_order={act_order}", flush=True)
+    layer = make_layer(k, n, group, dtype, act_order=act_order, seed=21, bits=8)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).to(dtype).to(dev)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    ks = torch.randint(0, k, (m,), generator=torch.Generator().manual_seed(4))
+    hot = torch.zeros(m, k, dtype=dtype)
+    hot[torch.arange(m), ks] = 1.0
+    out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_linear_kernel_w8(dev):
     from vllm_amd.mixed_precision import MarlinLinearKernel, MPLinearLayerConfig, choose_mp_linear_kernel
     from vllm_amd.scalar_type import scalar_types

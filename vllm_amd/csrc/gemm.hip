@@ -117,6 +117,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   const bool general_only = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3 ||
                             a->wtype == W4A16_WTYPE_FE2M1 ||
                             (a->flags & W4A16_F_ZP_FLOAT) != 0;
+  // ... except that the prefill kernel also has 8-bit (uint8b128, fp8) instantiations
+  const bool w8 = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3;
+  const bool fat_ok = !general_only || (w8 && !(a->flags & W4A16_F_ZP_FLOAT));
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
@@ -151,7 +154,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // 0.75 with one workgroup per compute unit and 1.15 per pair with two.  (2048 x 4096: 128 tiles of 128 rows leave
   // half the compute units idle, 256 tiles of 64 rows do not: 99 -> 75 us at K = 4096.)
   bool prefer_mid = false;
-  if (fat_tiles >= cus / 2 && forced_kind < 0) {
+  if (fat_tiles >= cus / 2 && forced_kind < 0 && !general_only) {
     const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
     const bool handoff = fat_tiles >= cus && tail > 0 && ceil_div(tail, mt128) * ceil_div(a->size_m, 64) <= cus;
     const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.7 : 1.0);
@@ -159,7 +162,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     const double mid_units = 1.15 * (double)(mid_tiles / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.75 : 1.15);
     prefer_mid = mid_units < 0.95 * fat_units;
   }
-  if (!moe && !general_only && pow2_group && a->size_m >= 128 && !prefer_mid && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
+  if (!moe && fat_ok && pow2_group && a->size_m >= 128 && !prefer_mid && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
     pl.kind = 2;
     pl.tn = 512;
@@ -180,7 +183,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     {
       const int64_t rounds = tiles / cus, tail = tiles - rounds * cus;
       const int64_t strips = ceil_div(tail, (int64_t)pl.mtiles);
-      if (rounds >= 1 && tail > 0 && strips < pl.ncp && strips * ceil_div(a->size_m, 64) <= cus && forced_kind != 2)
+      if (rounds >= 1 && tail > 0 && strips < pl.ncp && strips * ceil_div(a->size_m, 64) <= cus && forced_kind != 2 &&
+          !general_only)  // (the 64-row kernel is 4-bit only)
         pl.tail_strips = (int)strips;
     }
     return 0;

@@ -255,6 +255,39 @@ __device__ __forceinline__ void dequant_pair8(uint32_t xa0, uint32_t xa1, uint32
   }
 }
 
+// One register (J = 0..7, as dequant_piece) of what dequant_pair8 / dequant_pair8_fp8 produce, for the prefill kernel.
+// x0 / x1: the word of column half 0 / 1 of the k-tile that register J draws on (Q < 2: k-tile a, else b).
+template <int DT, bool UNIT_SCALE, bool FP8, int J>
+__device__ __forceinline__ uint32_t dequant_piece8(uint32_t x0, uint32_t x1, uint32_t s_pair) {
+  constexpr int HF = J >> 2, Q = J & 3;
+  const uint32_t x = HF ? x1 : x0;
+  if constexpr (FP8) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    float sf = 1.0f;
+    if (!UNIT_SCALE)
+      sf = ((DT == DT_F16) ? (HF ? f16_hi_f32(s_pair) : f16_lo_f32(s_pair))
+                           : (HF ? bf16_hi_f32(s_pair) : bf16_lo_f32(s_pair))) *
+           ((DT == DT_F16) ? 0x1.0p-8f : 0x1.0p-120f);
+    // bytes (k0, k0+8, k0+1, k0+9): register Q & 1 = 0 pairs (k0, k0+1), 1 pairs (k0+8, k0+9)
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)x, false);
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)x, true);
+    const float lo = (Q & 1) ? a.y : a.x, hi = (Q & 1) ? b.y : b.x;
+    return DT == DT_F16 ? pack_f16(lo * sf, hi * sf) : pack_bf16(lo * sf, hi * sf);
+  } else if constexpr (DT == DT_F16) {
+    uint32_t EX = 0x64006400u;
+    asm("" : "+v"(EX));
+    const f16x2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const uint32_t y = (Q & 1) ? (x >> 8) : x;
+    const f16x2 v = as_h2((y & 0x00ff00ffu) | EX) - bias;
+    const f16x2 s = as_h2(s_pair);
+    return as_u32(UNIT_SCALE ? v : v * (HF ? f16x2{s.y, s.y} : f16x2{s.x, s.x}));
+  } else {
+    const float sf = UNIT_SCALE ? 1.0f : (HF ? bf16_hi_f32(s_pair) : bf16_lo_f32(s_pair));
+    const float cf = -128.0f * sf;
+    return pack_bf16(__builtin_fmaf(ubyte_f32<(Q & 1)>(x), sf, cf), __builtin_fmaf(ubyte_f32<(Q & 1) + 2>(x), sf, cf));
+  }
+}
+
 // fp8 (OCP e4m3fn) weights in the 8-bit Marlin layout.  The scales the op receives carry the exponent offset the
 // reference folds into them at load time (marlin_utils_fp8.py:25-37: s * 2^8 for fp16, s * 2^120 for bf16, because
 // its kernel moves the fp8 bits into the 16-bit format without re-biasing the exponent, dequant.h:320-373).  Here the

@@ -27,8 +27,12 @@ constexpr int FB_D = 4;      // weight k-steps in flight per wavefront
 constexpr int FB_ABUF = 2 * FB_MB * 64 * 16;  // bytes of one A buffer: 2 k-steps x 8 m-blocks x 64 lanes x 16 B
 constexpr int FB_SMEM = (2 * FB_ABUF > 4 * 16 * RED_RS * 4) ? 2 * FB_ABUF : 4 * 16 * RED_RS * 4;
 
-template <int DT, bool ZP, bool CHANNEL>
+// BITS = 8: uint8b128 or (FP8) float8_e4m3fn weights in the 8-bit Marlin layout: twice the words per lane, the same 64
+// MFMAs per k-step; no zero points.
+template <int DT, bool ZP, bool CHANNEL, int BITS = 4, bool FP8 = false>
 __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
+  static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights have no zero points");
+  static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
   const int t = threadIdx.x;
@@ -45,8 +49,9 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
 
   // ---- weights of this wavefront
   const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
-  const int64_t b_row = p.N >> 1;
-  const u32x4* bp = (const u32x4*)p.B + nt * 32 + (4 * c + g);
+  // 4-bit: 32 u32x4 per n-tile and k-tile, one per Marlin thread; 8-bit: 64, two per thread (words 2w + half)
+  const int64_t b_row = (BITS == 4) ? (p.N >> 1) : p.N;
+  const u32x4* bp = (const u32x4*)p.B + nt * (8 * BITS) + (4 * c + g) * (BITS / 4);
   const int64_t s_row = p.N >> 3;
   const u32x4* sp = (const u32x4*)p.S + nt * 8 + c;
   const uint32_t* zp = ZP ? p.Z + nt * 8 + c : nullptr;
@@ -88,6 +93,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
 
   struct Stage {
     u32x4 b0, b1, sc;
+    u32x4 b0h, b1h;  // 8-bit weights only: the thread's words 2, 3
     uint32_t zq;
   };
   Stage st[FB_D];
@@ -99,6 +105,16 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+    if constexpr (BITS == 8) {
+      s.b0h = bp[(int64_t)(2 * ks) * b_row + 1];
+      s.b1h = bp[(int64_t)(2 * ks + 1) * b_row + 1];
+    }
+  };
+  // 8-bit: the words of Marlin word position w are elements 2(w & 1) [column half 0] and 2(w & 1) + 1 [half 1] of
+  // the thread's first (w < 2) or second 16 bytes, per k-tile
+  auto word8 = [&](const Stage& s, int w, int ktile, int half) -> uint32_t {
+    const u32x4& v = ktile == 0 ? (w < 2 ? s.b0 : s.b0h) : (w < 2 ? s.b1 : s.b1h);
+    return v[2 * (w & 1) + half];
   };
   auto col_const = [&](const Stage& s, int w) {
     uint32_t z0 = 8, z1 = 8;
@@ -130,8 +146,16 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   u32x4 ob[2][4][2];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    const ColConst<DT> cc = col_const(st[0], w);
-    dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], cc, ob[0][w][0], ob[0][w][1]);
+    if constexpr (BITS == 4) {
+      const ColConst<DT> cc = col_const(st[0], w);
+      dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], cc, ob[0][w][0], ob[0][w][1]);
+    } else if constexpr (FP8) {
+      dequant_pair8_fp8<DT, UNIT>(word8(st[0], w, 0, 0), word8(st[0], w, 0, 1), word8(st[0], w, 1, 0),
+                                  word8(st[0], w, 1, 1), CHANNEL ? 0u : st[0].sc[w], ob[0][w][0], ob[0][w][1]);
+    } else {
+      dequant_pair8<DT, UNIT>(word8(st[0], w, 0, 0), word8(st[0], w, 0, 1), word8(st[0], w, 1, 0),
+                              word8(st[0], w, 1, 1), CHANNEL ? 0u : st[0].sc[w], ob[0][w][0], ob[0][w][1]);
+    }
   }
   __syncthreads();
 
@@ -153,7 +177,12 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
         constexpr int J = decltype(j_tag)::value;
         mfma_inplace<DT>(acc[J][w][0], af[J], ob[CUR][w][0]);
         mfma_inplace<DT>(acc[J][w][1], af[J], ob[CUR][w][1]);
-        const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        uint32_t r;
+        if constexpr (BITS == 4)
+          r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        else
+          r = dequant_piece8<DT, UNIT, FP8, J>(word8(nxt, w, (J & 3) >> 1, 0), word8(nxt, w, (J & 3) >> 1, 1),
+                                               CHANNEL ? 0u : nxt.sc[w]);
         if constexpr (J < 4)
           ob[CUR ^ 1][w][0][J] = r;
         else
@@ -218,7 +247,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     for (int j = 0; j < 4; ++j) {
       if (CHANNEL) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+        cs[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (FP8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
       if (bias) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
@@ -262,10 +291,22 @@ static fat_fn pick_fat2(bool zp, bool channel) {
   if (zp) return channel ? fat_kernel<DT, true, true> : fat_kernel<DT, true, false>;
   return channel ? fat_kernel<DT, false, true> : fat_kernel<DT, false, false>;
 }
+template <int DT>
+static fat_fn pick_fat8(bool fp8, bool channel) {
+  if (fp8) return channel ? fat_kernel<DT, false, true, 8, true> : fat_kernel<DT, false, false, 8, true>;
+  return channel ? fat_kernel<DT, false, true, 8, false> : fat_kernel<DT, false, false, 8, false>;
+}
 
 int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
-  const bool zp = a->b_zeros != nullptr;
-  fat_fn fn = a->dtype == DT_F16 ? pick_fat2<DT_F16>(zp, pl.gm == GM_CHANNEL) : pick_fat2<DT_BF16>(zp, pl.gm == GM_CHANNEL);
+  const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
+  fat_fn fn;
+  if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
+    const bool fp8 = a->wtype == W4A16_WTYPE_FE4M3;
+    if (zp) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    fn = a->dtype == DT_F16 ? pick_fat8<DT_F16>(fp8, channel) : pick_fat8<DT_BF16>(fp8, channel);
+  } else {
+    fn = a->dtype == DT_F16 ? pick_fat2<DT_F16>(zp, channel) : pick_fat2<DT_BF16>(zp, channel);
+  }
   KParams p = make_kparams(a, pl);
   const int64_t grid = (int64_t)pl.tiles;
   if (grid <= 0) return 0;
