@@ -78,6 +78,25 @@ def test_reference_grid(ops, dev, workspace, kind, dtype, n_chunk, mnk):
     assert float((out.float() - ref).abs().mean() / ref.abs().mean()) < 0.04
 
 
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("nvfp4", torch.bfloat16), ("mxfp4", torch.bfloat16)])
+def test_prefill_tiles(ops, dev, workspace, kind, dtype):
+    """Enough 128-row tiles for the prefill kernel, with a partial row tile and a partial 512-column strip: random
+    activations against the oracle, one-hot rows bit-exact."""
+    size_m, size_k, size_n = 1100, 512, 8256
+    print(f"fp4 prefill {kind} dtype={dtype}", flush=True)
+    w, _, mq, ms, gs = make(kind, size_k, size_n, dtype, dev, 9)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).to(dtype)
+    out = run(ops, a.to(dev), mq, ms, gs, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w))
+    assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, gs, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_linear_helpers_and_bias(ops, dev, workspace):
     from vllm_amd import marlin_utils_fp4 as f4
     from vllm_amd.marlin_utils import marlin_permute_bias

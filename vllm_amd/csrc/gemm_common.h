@@ -431,6 +431,19 @@ __device__ __forceinline__ void dequant_pair_nvfp4_f16_direct(uint32_t xa, uint3
   o1 = u32x4{m(cvt_fp4x2<DT_F16, 1>(xa, pre), sa1), m(cvt_fp4x2<DT_F16, 3>(xa, pre), sa1),
              m(cvt_fp4x2<DT_F16, 1>(xb, pre), sb1), m(cvt_fp4x2<DT_F16, 3>(xb, pre), sb1)};
 }
+// One register (J = 0..7, as dequant_piece) of what dequant_pair_fp4 produces, for the prefill kernel.  x: the word of
+// the k-tile register J draws on; s0 / s1: that k-tile's true scale for column half 0 / 1.
+template <int DT, int J>
+__device__ __forceinline__ uint32_t dequant_piece_fp4(uint32_t x, float s0, float s1) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  constexpr int HF = J >> 2, Q = J & 3;
+  const float sf = HF ? s1 : s0;
+  // bytes 0, 1: K rows (k0, k0+8) of columns n0, n0+8; bytes 2, 3: rows (k0+1, k0+9)
+  const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, HF);
+  const f32x2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(x, 1.0f, HF + 2);
+  const float lo = (Q & 1) ? a.y : a.x, hi = (Q & 1) ? b.y : b.x;
+  return DT == DT_F16 ? pack_f16(lo * sf, hi * sf) : pack_bf16(lo * sf, hi * sf);
+}
 // Scale bytes of Marlin word w in a lane's 16-byte fp4 scale record: 8 bytes per k-tile (NVFP4) or k-step (MXFP4),
 // stored in the order (e0, e2, e1, e3, e4, e6, e5, e7) with e = 2w + half (marlin_utils_fp4.py:44-47, 68-71).
 // half_rec: the 8 bytes as two dwords; returns byte of column half 0 in bits 0..7 and of half 1 in bits 16..23.

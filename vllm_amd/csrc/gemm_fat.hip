@@ -29,10 +29,13 @@ constexpr int FB_SMEM = (2 * FB_ABUF > 4 * 16 * RED_RS * 4) ? 2 * FB_ABUF : 4 * 
 
 // BITS = 8: uint8b128 or (FP8) float8_e4m3fn weights in the 8-bit Marlin layout: twice the words per lane, the same 64
 // MFMAs per k-step; no zero points.
-template <int DT, bool ZP, bool CHANNEL, int BITS = 4, bool FP8 = false>
+// FP4 = 1 / 2: float4_e2m1f weights (4-bit layout) with NVFP4 / MXFP4 scale records, one 16-byte record per lane and
+// k-step / two k-steps (the host sets the group to 1 / 2 k-steps); NVFP4's global scale is applied to the accumulator.
+template <int DT, bool ZP, bool CHANNEL, int BITS = 4, bool FP8 = false, int FP4 = 0>
 __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights have no zero points");
   static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
+  static_assert(FP4 == 0 || (BITS == 4 && !ZP && !CHANNEL), "fp4 weights: grouped scale records, no zero points");
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
   const int t = threadIdx.x;
@@ -103,12 +106,26 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     if (!CHANNEL) gi = ks >> p.group_shift;  // the host only picks this kernel for power-of-two group sizes
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
     if constexpr (BITS == 8) {
       s.b0h = bp[(int64_t)(2 * ks) * b_row + 1];
       s.b1h = bp[(int64_t)(2 * ks + 1) * b_row + 1];
     }
+  };
+  struct Fp4Scales { float a0, a1, b0, b1; };
+  auto fp4_scales = [&](const Stage& s, int w) {
+    Fp4Scales r{1.f, 1.f, 1.f, 1.f};
+    if constexpr (FP4 == 1) {
+      const uint32_t ba = fp4_scale_bytes(s.sc[0], s.sc[1], w), bb = fp4_scale_bytes(s.sc[2], s.sc[3], w);
+      r = Fp4Scales{nvfp4_scale_f32(ba & 0xff), nvfp4_scale_f32(ba >> 16), nvfp4_scale_f32(bb & 0xff), nvfp4_scale_f32(bb >> 16)};
+    } else if constexpr (FP4 == 2) {
+      const uint32_t bs = s.zq ? fp4_scale_bytes(s.sc[2], s.sc[3], w) : fp4_scale_bytes(s.sc[0], s.sc[1], w);
+      const float s0 = mxfp4_scale_f32(bs & 0xff), s1 = mxfp4_scale_f32(bs >> 16);
+      r = Fp4Scales{s0, s1, s0, s1};
+    }
+    return r;
   };
   // 8-bit: the words of Marlin word position w are elements 2(w & 1) [column half 0] and 2(w & 1) + 1 [half 1] of
   // the thread's first (w < 2) or second 16 bytes, per k-tile
@@ -146,7 +163,10 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   u32x4 ob[2][4][2];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    if constexpr (BITS == 4) {
+    if constexpr (FP4 != 0) {
+      const Fp4Scales fs = fp4_scales(st[0], w);
+      dequant_pair_fp4<DT>(st[0].b0[w], st[0].b1[w], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][w][0], ob[0][w][1]);
+    } else if constexpr (BITS == 4) {
       const ColConst<DT> cc = col_const(st[0], w);
       dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], cc, ob[0][w][0], ob[0][w][1]);
     } else if constexpr (FP8) {
@@ -172,13 +192,16 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     auto word = [&](auto w_tag) {
       constexpr int w = decltype(w_tag)::value;
       const ColConst<DT> cc = col_const(nxt, w);
+      const Fp4Scales fs = fp4_scales(nxt, w);
       const uint32_t xa = nxt.b0[w], xb = nxt.b1[w];
       auto step = [&](auto j_tag) {
         constexpr int J = decltype(j_tag)::value;
         mfma_inplace<DT>(acc[J][w][0], af[J], ob[CUR][w][0]);
         mfma_inplace<DT>(acc[J][w][1], af[J], ob[CUR][w][1]);
         uint32_t r;
-        if constexpr (BITS == 4)
+        if constexpr (FP4 != 0)
+          r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
+        else if constexpr (BITS == 4)
           r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
         else
           r = dequant_piece8<DT, UNIT, FP8, J>(word8(nxt, w, (J & 3) >> 1, 0), word8(nxt, w, (J & 3) >> 1, 1),
@@ -241,6 +264,13 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   const int ncol = cp * 128 + fc4;
   const bool fcol_ok = wave_on && ncol < p.N;
   float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (FP4 == 1) {
+    // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
+    const uint16_t gv = *(const uint16_t*)p.gscale;
+    const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cs[j] = gs;
+  }
   if (fcol_ok) {
     const int base = ncol & ~31, cl = ncol & 31;
 #pragma unroll
@@ -300,7 +330,12 @@ static fat_fn pick_fat8(bool fp8, bool channel) {
 int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   fat_fn fn;
-  if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
+  if (a->wtype == W4A16_WTYPE_FE2M1) {
+    if (zp || channel) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    fn = a->global_scale ? (a->dtype == DT_F16 ? fat_kernel<DT_F16, false, false, 4, false, 1>
+                                               : fat_kernel<DT_BF16, false, false, 4, false, 1>)
+                         : fat_kernel<DT_BF16, false, false, 4, false, 2>;
+  } else if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
     const bool fp8 = a->wtype == W4A16_WTYPE_FE4M3;
     if (zp) return fail(W4A16_EINVAL, "unsupported kernel variant");
     fn = a->dtype == DT_F16 ? pick_fat8<DT_F16>(fp8, channel) : pick_fat8<DT_BF16>(fp8, channel);
