@@ -86,6 +86,24 @@ def test_llama_shape_decode_and_prefill_rows(ops, dev, workspace):
         assert m["max_rel"] <= 2e-2 and m["mean_rel"] < 0.04, (size_m, m)
 
 
+def test_prefill_tiles(ops, dev, workspace):
+    """Enough 128-row tiles for the prefill kernel, with a partial row tile and a partial 512-column strip: random
+    activations against the oracle, one-hot rows bit-exact."""
+    size_m, size_k, size_n = 1100, 512, 8256
+    _, _, _, mq, ms, mz = make_hqq(size_k, size_n, 13)
+    w = gr.dequant_marlin_float_zp(mq, ms, mz, size_k, size_n)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).half()
+    out = run(ops, a.to(dev), mq, ms, mz, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w))
+    assert m["max_rel"] <= 2e-2 and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=torch.float16)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, mz, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_argument_errors(ops, dev, workspace):
     import vllm_amd.scalar_type as vst
     size_k, size_n = 256, 128

@@ -180,6 +180,28 @@ __device__ __forceinline__ void dequant_pair_zpf(uint32_t xa, uint32_t xb, uint3
   o1 = u32x4{lo(ya, s1, nz1), hi(ya, s1, nz1), lo(yb, s1, nz1), hi(yb, s1, nz1)};
 }
 
+// One register (J = 0..7, as dequant_piece) of what dequant_pair_zpf produces, for the prefill kernel.
+template <int J>
+__device__ __forceinline__ uint32_t dequant_piece_zpf(uint32_t xa, uint32_t xb, uint32_t s_pair, uint32_t zs_pair) {
+  constexpr int HF = J >> 2, Q = J & 3;
+  uint32_t EX = 0x64006400u;
+  asm("" : "+v"(EX));
+  const uint32_t x = (Q < 2) ? xa : xb;
+  const uint32_t y = HF ? (x >> 8) : x;
+  const f16x2 s = as_h2(s_pair), zs = as_h2(zs_pair);
+  const f16x2 sc = HF ? f16x2{s.y, s.y} : f16x2{s.x, s.x};
+  const f16x2 nz = HF ? f16x2{-zs.y, -zs.y} : f16x2{-zs.x, -zs.x};
+  f16x2 q;
+  if constexpr ((Q & 1) == 0) {
+    const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    q = as_h2((y & 0x000f000fu) | EX) - k1024;
+  } else {
+    const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f}, k64 = {(_Float16)64.0f, (_Float16)64.0f};
+    q = as_h2((y & 0x00f000f0u) | EX) * sixteenth - k64;
+  }
+  return as_u32(__builtin_elementwise_fma(q, sc, nz));
+}
+
 // byte N of x as float (v_cvt_f32_ubyteN; the compiler only finds the byte-0 form on its own)
 template <int N>
 __device__ __forceinline__ float ubyte_f32(uint32_t x) {

@@ -31,8 +31,10 @@ constexpr int FB_SMEM = (2 * FB_ABUF > 4 * 16 * RED_RS * 4) ? 2 * FB_ABUF : 4 * 
 // MFMAs per k-step; no zero points.
 // FP4 = 1 / 2: float4_e2m1f weights (4-bit layout) with NVFP4 / MXFP4 scale records, one 16-byte record per lane and
 // k-step / two k-steps (the host sets the group to 1 / 2 k-steps); NVFP4's global scale is applied to the accumulator.
-template <int DT, bool ZP, bool CHANNEL, int BITS = 4, bool FP8 = false, int FP4 = 0>
+// ZPF: uint4 weights with fp16 zero points laid out like the scales (HQQ): operand = fma(q, s, -half(zp * s)).
+template <int DT, bool ZP, bool CHANNEL, int BITS = 4, bool FP8 = false, int FP4 = 0, bool ZPF = false>
 __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
+  static_assert(!ZPF || (DT == DT_F16 && !ZP && !CHANNEL && BITS == 4 && FP4 == 0), "float zero points: fp16 uint4 grouped");
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights have no zero points");
   static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
   static_assert(FP4 == 0 || (BITS == 4 && !ZP && !CHANNEL), "fp4 weights: grouped scale records, no zero points");
@@ -58,6 +60,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   const int64_t s_row = p.N >> 3;
   const u32x4* sp = (const u32x4*)p.S + nt * 8 + c;
   const uint32_t* zp = ZP ? p.Z + nt * 8 + c : nullptr;
+  const u32x4* zfp = ZPF ? (const u32x4*)p.Z + nt * 8 + c : nullptr;  // fp16 zero points: indexed like the scales
 
   // ---- activation staging: thread t loads piece (t & 7) of rows (t >> 3) + 32 i, i = 0..3
   const int piece = t & 7;
@@ -97,6 +100,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   struct Stage {
     u32x4 b0, b1, sc;
     u32x4 b0h, b1h;  // 8-bit weights only: the thread's words 2, 3
+    u32x4 zf;        // float zero points only
     uint32_t zq;
   };
   Stage st[FB_D];
@@ -107,6 +111,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
+    if (ZPF) s.zf = zfp[(int64_t)gi * s_row];
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
     if constexpr (BITS == 8) {
@@ -163,7 +168,10 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   u32x4 ob[2][4][2];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    if constexpr (FP4 != 0) {
+    if constexpr (ZPF) {
+      dequant_pair_zpf(st[0].b0[w], st[0].b1[w], st[0].sc[w], as_u32(as_h2(st[0].zf[w]) * as_h2(st[0].sc[w])),
+                       ob[0][w][0], ob[0][w][1]);
+    } else if constexpr (FP4 != 0) {
       const Fp4Scales fs = fp4_scales(st[0], w);
       dequant_pair_fp4<DT>(st[0].b0[w], st[0].b1[w], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][w][0], ob[0][w][1]);
     } else if constexpr (BITS == 4) {
@@ -193,13 +201,17 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
       constexpr int w = decltype(w_tag)::value;
       const ColConst<DT> cc = col_const(nxt, w);
       const Fp4Scales fs = fp4_scales(nxt, w);
+      uint32_t zs = 0;
+      if constexpr (ZPF) zs = as_u32(as_h2(nxt.zf[w]) * as_h2(nxt.sc[w]));
       const uint32_t xa = nxt.b0[w], xb = nxt.b1[w];
       auto step = [&](auto j_tag) {
         constexpr int J = decltype(j_tag)::value;
         mfma_inplace<DT>(acc[J][w][0], af[J], ob[CUR][w][0]);
         mfma_inplace<DT>(acc[J][w][1], af[J], ob[CUR][w][1]);
         uint32_t r;
-        if constexpr (FP4 != 0)
+        if constexpr (ZPF)
+          r = dequant_piece_zpf<J>(xa, xb, nxt.sc[w], zs);
+        else if constexpr (FP4 != 0)
           r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
         else if constexpr (BITS == 4)
           r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
@@ -330,7 +342,10 @@ static fat_fn pick_fat8(bool fp8, bool channel) {
 int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   fat_fn fn;
-  if (a->wtype == W4A16_WTYPE_FE2M1) {
+  if (a->flags & W4A16_F_ZP_FLOAT) {
+    if (a->dtype != DT_F16 || channel) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    fn = fat_kernel<DT_F16, false, false, 4, false, 0, true>;
+  } else if (a->wtype == W4A16_WTYPE_FE2M1) {
     if (zp || channel) return fail(W4A16_EINVAL, "unsupported kernel variant");
     fn = a->global_scale ? (a->dtype == DT_F16 ? fat_kernel<DT_F16, false, false, 4, false, 1>
                                                : fat_kernel<DT_BF16, false, false, 4, false, 1>)
