@@ -97,6 +97,24 @@ def test_prefill_tiles(ops, dev, workspace, kind, dtype):
     assert int(workspace.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("mxfp4", torch.bfloat16)])
+def test_64_row_tiles_with_split_k(ops, dev, workspace, kind, dtype):
+    """136 tiles of 64 x 512: the 64-row kernel splits K in two and a second kernel adds the partial tiles (and applies
+    NVFP4's global scale)."""
+    size_m, size_k, size_n = 512, 2048, 8704
+    w, _, mq, ms, gs = make(kind, size_k, size_n, dtype, dev, 23)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).to(dtype)
+    out = run(ops, a.to(dev), mq, ms, gs, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w))
+    assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, gs, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_linear_helpers_and_bias(ops, dev, workspace):
     from vllm_amd import marlin_utils_fp4 as f4
     from vllm_amd.marlin_utils import marlin_permute_bias

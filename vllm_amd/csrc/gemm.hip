@@ -120,6 +120,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // ... except that the prefill kernel also has 8-bit (uint8b128, fp8), fp4 and float-zero-point instantiations
   const bool w8 = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3;
   const bool fat_ok = !general_only || w8 || a->wtype == W4A16_WTYPE_FE2M1 || (a->flags & W4A16_F_ZP_FLOAT);
+  const bool mid_ok = !general_only || a->wtype == W4A16_WTYPE_FE2M1;  // the 64-row kernel: 4-bit integers and fp4
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
@@ -154,7 +155,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // 0.75 with one workgroup per compute unit and 1.15 per pair with two.  (2048 x 4096: 128 tiles of 128 rows leave
   // half the compute units idle, 256 tiles of 64 rows do not: 99 -> 75 us at K = 4096.)
   bool prefer_mid = false;
-  if (fat_tiles >= cus / 2 && forced_kind < 0 && !general_only) {
+  if (fat_tiles >= cus / 2 && forced_kind < 0 && mid_ok) {
     const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
     const bool handoff = fat_tiles >= cus && tail > 0 && ceil_div(tail, mt128) * ceil_div(a->size_m, 64) <= cus;
     const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.7 : 1.0);
@@ -184,7 +185,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       const int64_t rounds = tiles / cus, tail = tiles - rounds * cus;
       const int64_t strips = ceil_div(tail, (int64_t)pl.mtiles);
       if (rounds >= 1 && tail > 0 && strips < pl.ncp && strips * ceil_div(a->size_m, 64) <= cus && forced_kind != 2 &&
-          !general_only)  // (the 64-row kernel is 4-bit only)
+          mid_ok)
         pl.tail_strips = (int)strips;
     }
     return 0;
@@ -209,7 +210,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     int kps = (int)ceil_div(pl.total_ksteps, sp);
     kps = (kps + 3) / 4 * 4;
     sp = (int)ceil_div(pl.total_ksteps, kps);
-    const bool mid_shape = !general_only && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+    const bool mid_shape = mid_ok && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
                            (moe ? a->moe_block_size == 64
                                 : (a->size_m > 32 && mid_tiles >= cus / 2));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {

@@ -32,8 +32,11 @@ constexpr int MD_ABUF = 2 * MD_MB * 64 * 16;            // one A buffer: 2 k-ste
 constexpr int MD_SLABS = 4 * 16 * RED_RS * 4;           // four wavefront slabs of the epilogue
 constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_BM * 4;  // + C row of each tile row
 
-template <int DT, bool ZP, bool CHANNEL, bool MOE>
+// FP4 = 1 / 2: float4_e2m1f weights with NVFP4 / MXFP4 scale records (one 16-byte record per lane and k-step / two
+// k-steps); NVFP4's per-expert global scale is applied to the accumulator.
+template <int DT, bool ZP, bool CHANNEL, bool MOE, int FP4 = 0>
 __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
+  static_assert(FP4 == 0 || (!ZP && !CHANNEL), "fp4 weights: grouped scale records, no zero points");
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
   int* s_crow = (int*)(smem + MD_SMEM - MD_BM * 4);
@@ -57,12 +60,14 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint32_t* Zp = p.Z;
   const uint16_t* bias = (const uint16_t*)p.bias;
+  const uint16_t* gscale = (const uint16_t*)p.gscale;
   if (MOE) {
     if (row0 >= *p.ntpp) return;
     const int e = p.expert_ids[mt];
     if (e < 0) return;  // expert of another rank
     Bq += e * p.b_estride;
     Sc += e * p.s_estride;
+    if (FP4 == 1) gscale += e;
     if (ZP) Zp += e * p.z_estride;
     if (bias) bias += e * p.n_estride;
   }
@@ -143,8 +148,22 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     if (!CHANNEL) gi = ks >> p.group_shift;  // the host only picks this kernel for power-of-two group sizes
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+  };
+  struct Fp4Scales { float a0, a1, b0, b1; };  // k-tile a / b, column half 0 / 1
+  auto fp4_scales = [&](const Stage& s, int w) {
+    Fp4Scales r{1.f, 1.f, 1.f, 1.f};
+    if constexpr (FP4 == 1) {
+      const uint32_t ba = fp4_scale_bytes(s.sc[0], s.sc[1], w), bb = fp4_scale_bytes(s.sc[2], s.sc[3], w);
+      r = Fp4Scales{nvfp4_scale_f32(ba & 0xff), nvfp4_scale_f32(ba >> 16), nvfp4_scale_f32(bb & 0xff), nvfp4_scale_f32(bb >> 16)};
+    } else if constexpr (FP4 == 2) {
+      const uint32_t bs = s.zq ? fp4_scale_bytes(s.sc[2], s.sc[3], w) : fp4_scale_bytes(s.sc[0], s.sc[1], w);
+      const float s0 = mxfp4_scale_f32(bs & 0xff), s1 = mxfp4_scale_f32(bs >> 16);
+      r = Fp4Scales{s0, s1, s0, s1};
+    }
+    return r;
   };
   auto col_const = [&](const Stage& s, int w) {
     uint32_t z0 = 8, z1 = 8;
@@ -173,7 +192,10 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   store_a(0);
   // B operands of two Marlin words: the one whose MFMAs are being issued and the one being dequantised
   u32x4 ob[2][2];
-  {
+  if constexpr (FP4 != 0) {
+    const Fp4Scales fs = fp4_scales(st[0], 0);
+    dequant_pair_fp4<DT>(st[0].b0[0], st[0].b1[0], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][0], ob[0][1]);
+  } else {
     const ColConst<DT> cc = col_const(st[0], 0);
     dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], cc, ob[0][0], ob[0][1]);
   }
@@ -192,11 +214,16 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       constexpr int wn = (w + 1) & 3;
       const Stage& src = w == 3 ? nxt : cur;
       const ColConst<DT> cc = col_const(src, wn);
+      const Fp4Scales fs = fp4_scales(src, wn);
       const uint32_t xa = src.b0[wn], xb = src.b1[wn];
       auto step = [&](auto j_tag) {
         constexpr int J = decltype(j_tag)::value;
         mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
-        const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        uint32_t r;
+        if constexpr (FP4 != 0)
+          r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
+        else
+          r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
         if constexpr (J < 4)
           ob[wn & 1][0][J] = r;
         else
@@ -252,6 +279,13 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const int ncol = cp * 128 + fc4;
   const bool fcol_ok = wave_on && ncol < p.N;
   float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (FP4 == 1) {
+    // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
+    const uint16_t gv = *gscale;
+    const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cs[j] = gs;
+  }
   if (fcol_ok) {
     const int base = ncol & ~31, cl = ncol & 31;
 #pragma unroll
@@ -319,17 +353,25 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   const int row0 = mt * MD_BM;
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint16_t* bias = (const uint16_t*)p.bias;
+  const uint16_t* gscale = (const uint16_t*)p.gscale;  // NVFP4 only, else null
   if (MOE) {
     if (row0 >= *p.ntpp) return;
     const int e = p.expert_ids[mt];
     if (e < 0) return;
     Sc += e * p.s_estride;
+    if (gscale) gscale += e;
     if (bias) bias += e * p.n_estride;
   }
   const int fc4 = (t & 127) * 4;
   const int ncol = nt4 * 512 + fc4;
   if (ncol >= p.N) return;
   float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if (gscale) {
+    const uint16_t gv = *gscale;
+    const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cs[j] = gs;
+  }
   {
     const int base = ncol & ~31, cl = ncol & 31;
 #pragma unroll
@@ -390,7 +432,16 @@ int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   mid_fn fn, red;
-  if (a->dtype == DT_F16) {
+  if (a->wtype == W4A16_WTYPE_FE2M1) {
+    if (zp || channel) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    if (a->global_scale)
+      fn = a->dtype == DT_F16 ? (moe ? mid_kernel<DT_F16, false, false, true, 1> : mid_kernel<DT_F16, false, false, false, 1>)
+                              : (moe ? mid_kernel<DT_BF16, false, false, true, 1> : mid_kernel<DT_BF16, false, false, false, 1>);
+    else
+      fn = moe ? mid_kernel<DT_BF16, false, false, true, 2> : mid_kernel<DT_BF16, false, false, false, 2>;
+    red = a->dtype == DT_F16 ? (moe ? pick_reduce<DT_F16, true>(false) : pick_reduce<DT_F16, false>(false))
+                             : (moe ? pick_reduce<DT_BF16, true>(false) : pick_reduce<DT_BF16, false>(false));
+  } else if (a->dtype == DT_F16) {
     fn = moe ? pick_mid2<DT_F16, true>(zp, channel) : pick_mid2<DT_F16, false>(zp, channel);
     red = moe ? pick_reduce<DT_F16, true>(channel) : pick_reduce<DT_F16, false>(channel);
   } else {
