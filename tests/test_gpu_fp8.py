@@ -105,6 +105,24 @@ def test_prefill_tiles(ops, dev, workspace, dtype, group):
     assert int(workspace.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dtype,group", [(torch.float16, -1), (torch.bfloat16, 128)])
+def test_64_row_tiles_with_split_k(ops, dev, workspace, dtype, group):
+    """136 tiles of 64 x 512: the 64-row kernel splits K in two and a second kernel adds the partial tiles (and, with
+    channel-wise scales, takes the exponent offset out of them)."""
+    size_m, size_k, size_n = 512, 2048, 8704
+    w_ref, _, mq, ms = make_fp8(size_k, size_n, group, dtype, 19)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).to(dtype)
+    out = run(ops, a.to(dev), mq, ms, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w_ref))
+    assert m["max_rel"] <= TOL[dtype] and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w_ref[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_host_helpers_match_the_oracle(ops, dev, workspace):
     """marlin_quant_fp8_torch (repack op + scale permutation + exponent offset) against the oracle's tensors, and
     apply_fp8_marlin_linear with a bias."""

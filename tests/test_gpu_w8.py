@@ -78,6 +78,22 @@ def test_prefill_tiles_w8(ops, dev, workspace, dtype, group, act_order):
     assert int(workspace.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dtype,group", [(torch.float16, 128), (torch.bfloat16, -1)])
+def test_64_row_tiles_with_split_k_w8(ops, dev, workspace, dtype, group):
+    """136 tiles of 64 x 512: the 64-row kernel splits K in two and a second kernel adds the partial tiles."""
+    m, k, n = 512, 2048, 8704
+    layer = make_layer(k, n, group, dtype, seed=22, bits=8)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).to(dtype).to(dev)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    ks = torch.randint(0, k, (m,), generator=torch.Generator().manual_seed(4))
+    hot = torch.zeros(m, k, dtype=dtype)
+    hot[torch.arange(m), ks] = 1.0
+    out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_linear_kernel_w8(dev):
     from vllm_amd.mixed_precision import MarlinLinearKernel, MPLinearLayerConfig, choose_mp_linear_kernel
     from vllm_amd.scalar_type import scalar_types

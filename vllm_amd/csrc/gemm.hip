@@ -120,7 +120,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // ... except that the prefill kernel also has 8-bit (uint8b128, fp8), fp4 and float-zero-point instantiations
   const bool w8 = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3;
   const bool fat_ok = !general_only || w8 || a->wtype == W4A16_WTYPE_FE2M1 || (a->flags & W4A16_F_ZP_FLOAT);
-  const bool mid_ok = !general_only || a->wtype == W4A16_WTYPE_FE2M1;  // the 64-row kernel: 4-bit integers and fp4
+  // the 64-row kernel: everything but float zero points (8-bit MoE weights with act-order are refused just below)
+  const bool mid_ok = !general_only || a->wtype == W4A16_WTYPE_FE2M1 || w8;
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
   if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
     return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
@@ -155,7 +156,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // 0.75 with one workgroup per compute unit and 1.15 per pair with two.  (2048 x 4096: 128 tiles of 128 rows leave
   // half the compute units idle, 256 tiles of 64 rows do not: 99 -> 75 us at K = 4096.)
   bool prefer_mid = false;
-  if (fat_tiles >= cus / 2 && forced_kind < 0 && mid_ok) {
+  if (fat_tiles >= cus / 2 && forced_kind < 0 && mid_ok && !w8) {  // (the unit costs below are the 4-bit kernels')
     const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
     const bool handoff = fat_tiles >= cus && tail > 0 && ceil_div(tail, mt128) * ceil_div(a->size_m, 64) <= cus;
     const double fat_units = (double)(fat_tiles / cus) + (tail == 0 ? 0.0 : handoff ? 0.7 : 1.0);

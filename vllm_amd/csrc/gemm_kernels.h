@@ -17,6 +17,7 @@ struct KParams {
   const int32_t* perm;
   const void* bias;
   const void* gscale;  // NVFP4 global scale (one element of the activation type per expert), else null
+  int fp8;             // weights are float8_e4m3fn (their stored scales carry an exponent offset)
   float* ctmp;
   int32_t* locks;
   int lock_stride;
@@ -110,6 +111,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.perm = pl.use_perm ? a->perm : nullptr;
   p.bias = a->b_bias;
   p.gscale = a->global_scale;
+  p.fp8 = a->wtype == W4A16_WTYPE_FE4M3;
   p.ctmp = a->c_tmp;
   p.locks = a->workspace;
   // counters of neighbouring tiles 16 bytes apart when the workspace is long enough (arrivals complete sooner)

@@ -34,9 +34,13 @@ constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_B
 
 // FP4 = 1 / 2: float4_e2m1f weights with NVFP4 / MXFP4 scale records (one 16-byte record per lane and k-step / two
 // k-steps); NVFP4's per-expert global scale is applied to the accumulator.
-template <int DT, bool ZP, bool CHANNEL, bool MOE, int FP4 = 0>
+// BITS = 8: uint8b128 or (FP8) float8_e4m3fn weights in the 8-bit Marlin layout; their stages hold twice the weight
+// registers, which still fits the two-workgroups-per-compute-unit budget (the grouped variants spill 2-9 registers).
+template <int DT, bool ZP, bool CHANNEL, bool MOE, int FP4 = 0, int BITS = 4, bool FP8 = false>
 __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
-  static_assert(FP4 == 0 || (!ZP && !CHANNEL), "fp4 weights: grouped scale records, no zero points");
+  static_assert(FP4 == 0 || (!ZP && !CHANNEL && BITS == 4), "fp4 weights: grouped scale records, no zero points");
+  static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights have no zero points");
+  static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
   int* s_crow = (int*)(smem + MD_SMEM - MD_BM * 4);
@@ -92,8 +96,9 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 
   // ---- weights of this wavefront
   const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
-  const int64_t b_row = p.N >> 1;
-  const u32x4* bp = (const u32x4*)Bq + nt * 32 + (4 * c + g);
+  // 4-bit: 32 u32x4 per n-tile and k-tile, one per Marlin thread; 8-bit: 64, two per thread (words 2w + half)
+  const int64_t b_row = (BITS == 4) ? (p.N >> 1) : p.N;
+  const u32x4* bp = (const u32x4*)Bq + nt * (8 * BITS) + (4 * c + g) * (BITS / 4);
   const int64_t s_row = p.N >> 3;
   const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
@@ -139,6 +144,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 
   struct Stage {
     u32x4 b0, b1, sc;
+    u32x4 b0h, b1h;  // 8-bit weights only: the thread's words 2, 3
     uint32_t zq;
   };
   Stage st[MD_D];
@@ -151,6 +157,16 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+    if constexpr (BITS == 8) {
+      s.b0h = bp[(int64_t)(2 * ks) * b_row + 1];
+      s.b1h = bp[(int64_t)(2 * ks + 1) * b_row + 1];
+    }
+  };
+  // 8-bit: the words of Marlin word position w are elements 2(w & 1) [column half 0] and 2(w & 1) + 1 [half 1] of
+  // the thread's first (w < 2) or second 16 bytes, per k-tile
+  auto word8 = [&](const Stage& s, int w, int ktile, int half) -> uint32_t {
+    const u32x4& v = ktile == 0 ? (w < 2 ? s.b0 : s.b0h) : (w < 2 ? s.b1 : s.b1h);
+    return v[2 * (w & 1) + half];
   };
   struct Fp4Scales { float a0, a1, b0, b1; };  // k-tile a / b, column half 0 / 1
   auto fp4_scales = [&](const Stage& s, int w) {
@@ -195,6 +211,12 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   if constexpr (FP4 != 0) {
     const Fp4Scales fs = fp4_scales(st[0], 0);
     dequant_pair_fp4<DT>(st[0].b0[0], st[0].b1[0], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][0], ob[0][1]);
+  } else if constexpr (FP8) {
+    dequant_pair8_fp8<DT, UNIT>(word8(st[0], 0, 0, 0), word8(st[0], 0, 0, 1), word8(st[0], 0, 1, 0), word8(st[0], 0, 1, 1),
+                                CHANNEL ? 0u : st[0].sc[0], ob[0][0], ob[0][1]);
+  } else if constexpr (BITS == 8) {
+    dequant_pair8<DT, UNIT>(word8(st[0], 0, 0, 0), word8(st[0], 0, 0, 1), word8(st[0], 0, 1, 0), word8(st[0], 0, 1, 1),
+                            CHANNEL ? 0u : st[0].sc[0], ob[0][0], ob[0][1]);
   } else {
     const ColConst<DT> cc = col_const(st[0], 0);
     dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], cc, ob[0][0], ob[0][1]);
@@ -222,6 +244,9 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
         uint32_t r;
         if constexpr (FP4 != 0)
           r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
+        else if constexpr (BITS == 8)
+          r = dequant_piece8<DT, UNIT, FP8, J>(word8(src, wn, (J & 3) >> 1, 0), word8(src, wn, (J & 3) >> 1, 1),
+                                               CHANNEL ? 0u : src.sc[wn]);
         else
           r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
         if constexpr (J < 4)
@@ -292,7 +317,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     for (int j = 0; j < 4; ++j) {
       if (CHANNEL) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+        cs[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
       if (bias) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
@@ -378,7 +403,7 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
     for (int j = 0; j < 4; ++j) {
       if (CHANNEL) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+        cs[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
       if (bias) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
@@ -424,6 +449,11 @@ static mid_fn pick_mid2(bool zp, bool channel) {
   return channel ? mid_kernel<DT, false, true, MOE> : mid_kernel<DT, false, false, MOE>;
 }
 template <int DT, bool MOE>
+static mid_fn pick_mid8(bool fp8, bool channel) {
+  if (fp8) return channel ? mid_kernel<DT, false, true, MOE, 0, 8, true> : mid_kernel<DT, false, false, MOE, 0, 8, true>;
+  return channel ? mid_kernel<DT, false, true, MOE, 0, 8, false> : mid_kernel<DT, false, false, MOE, 0, 8, false>;
+}
+template <int DT, bool MOE>
 static mid_fn pick_reduce(bool channel) {
   return channel ? mid_reduce_kernel<DT, true, MOE> : mid_reduce_kernel<DT, false, MOE>;
 }
@@ -432,7 +462,17 @@ int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   mid_fn fn, red;
-  if (a->wtype == W4A16_WTYPE_FE2M1) {
+  if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
+    if (zp) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    const bool fp8 = a->wtype == W4A16_WTYPE_FE4M3;
+    if (a->dtype == DT_F16) {
+      fn = moe ? pick_mid8<DT_F16, true>(fp8, channel) : pick_mid8<DT_F16, false>(fp8, channel);
+      red = moe ? pick_reduce<DT_F16, true>(channel) : pick_reduce<DT_F16, false>(channel);
+    } else {
+      fn = moe ? pick_mid8<DT_BF16, true>(fp8, channel) : pick_mid8<DT_BF16, false>(fp8, channel);
+      red = moe ? pick_reduce<DT_BF16, true>(channel) : pick_reduce<DT_BF16, false>(channel);
+    }
+  } else if (a->wtype == W4A16_WTYPE_FE2M1) {
     if (zp || channel) return fail(W4A16_EINVAL, "unsupported kernel variant");
     if (a->global_scale)
       fn = a->dtype == DT_F16 ? (moe ? mid_kernel<DT_F16, false, false, true, 1> : mid_kernel<DT_F16, false, false, false, 1>)
