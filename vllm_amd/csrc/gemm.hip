@@ -200,7 +200,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     const int64_t mid_tiles = mid_mtiles * ceil_div(a->size_n, 512);
     int sp = 1;
     // (measured: worth it from about cus/2 tiles up to 3/4 cus dense, up to cus for MoE, whose tile count is an upper bound)
-    if (mid_tiles >= cus / 2 && mid_tiles < (moe ? cus : cus * 3 / 4)) {
+    if ((mid_tiles >= cus / 2 || forced_kind == 3) && mid_tiles < (moe ? cus : cus * 3 / 4)) {
       const int by_k = pl.total_ksteps / 32;
       const int by_cus = (int)(2 * cus / mid_tiles);
       sp = by_k < by_cus ? by_k : by_cus;
@@ -213,7 +213,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     sp = (int)ceil_div(pl.total_ksteps, kps);
     const bool mid_shape = mid_ok && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
                            (moe ? a->moe_block_size == 64
-                                : (a->size_m > 32 && mid_tiles >= cus / 2));
+                                : (a->size_m > 32 && (mid_tiles >= cus / 2 || (forced_kind == 3 && mid_tiles >= cus / 16))));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
       W4A16_CHECK(mid_tiles * sp < (1LL << 31) / 64, "too many tiles");
       pl.kind = 3;
@@ -265,7 +265,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       const double bytes = (double)tiles * a->size_k * tn / 2.0;
       const double wg_rate = mb == 1 ? (tn == 64 ? 20e3 : 33e3) : mb == 2 ? 12e3 : 9e3;  // bytes per us
       const double chip_rate = 4.7e6;
-      const double t_xchg = 1.5;
+      const double t_xchg = 2.2;
       const int unit = decode_ok ? 16 : 8;  // k-steps per split needed to give every wavefront work
       const int max_splits = pl.total_ksteps / unit > 0 ? pl.total_ksteps / unit : 1;
       for (int sp = 1; sp <= 16; ++sp) {
@@ -275,11 +275,19 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
         const int64_t wgs = tiles * sp;
         if (sp > 1 && wgs > cus) break;
         const int64_t rounds = ceil_div(wgs, cus);
-        double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
-        if (rate > chip_rate) rate = chip_rate;
+        const double rate = (double)wgs / (double)rounds * wg_rate;  // workgroups resident at a time
         // the last workgroup of a tile re-reads every split's partial tile at about one workgroup's stream rate
         const double t_fix = sp > 1 ? t_xchg + sp * (double)(16 * mb * tn * 4) / 20e3 : 0.0;
-        const double t = bytes / rate + t_fix;
+        // HBM sees every weight byte once; further row tiles re-read the strips, from L2 at about twice that rate when
+        // the whole weight fits the eight 4 MB L2s (down_proj at 64 rows: 128-column tiles with two splits take 22 us,
+        // 64-column tiles without 27), else at the same rate again (gate_up: 2 row tiles cost 28 us, not 19)
+        const double unique = (double)ncol_tiles * a->size_k * tn / 2.0;
+        const double t_mem = unique / chip_rate + (bytes - unique) / (unique <= 32e6 ? 9.2e6 : chip_rate);
+        const double t_wg = bytes / rate;
+        const double t = (t_wg > t_mem ? t_wg : t_mem) + t_fix;
+        if (debug_plan >= 2)
+          fprintf(stderr, "[w4a16]   cand kind=%d tn=%d mb=%d tiles=%lld sp=%d: wg %.2f mem %.2f fix %.2f -> %.2f\n", decode_ok ? 1 : 0,
+                  tn, mb, (long long)tiles, sp, t_wg, t_mem, t_fix, t);
         if (t < best.t) best = Cand{decode_ok ? 1 : 0, tn, sp, mb, t};
       }
     }
