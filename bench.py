@@ -275,6 +275,49 @@ def bench_moe(ops, wtype, dev):
     return out
 
 
+def bench_other_types(ops, dev, workspace):
+    """The other weight types of the operator on gate_up (4096 x 28672): uint8b128, float8_e4m3fn, NVFP4, MXFP4 and
+    uint4 with fp16 zero points, at M = 16 and M = 4096 (warm weights, random codes; parity is the tests' business)."""
+    from vllm_amd import marlin_utils_fp4 as f4, marlin_utils_fp8 as f8
+    from vllm_amd.marlin_utils import marlin_permute_scales
+    from vllm_amd.scalar_type import scalar_types as st
+    k, n = LAYERS["gate_up"]
+    e = torch.empty(0, dtype=torch.int32, device=dev)
+    torch.manual_seed(0)
+    w16 = torch.randn(n, k, dtype=torch.float16, device=dev) * 0.02
+    cases = {}
+    q8 = torch.randint(-2**31, 2**31 - 1, (k // 16, 4 * n), dtype=torch.int32, device=dev)
+    s8 = marlin_permute_scales((torch.rand(k // GROUP, n, device=dev) * 0.01).half(), k, n, GROUP)
+    cases["uint8b128_f16_g128"] = (torch.float16, 1.0, lambda a: ops.gptq_marlin_gemm(
+        a, None, q8, None, s8, None, None, e, e, workspace, st.uint8b128, a.shape[0], n, k))
+    _, qf8, sf8 = f8.marlin_quant_fp8_torch(w16, GROUP)
+    cases["fp8_e4m3fn_f16_g128"] = (torch.float16, 1.0, lambda a: ops.gptq_marlin_gemm(
+        a, None, qf8, None, sf8, None, None, None, None, workspace, st.float8_e4m3fn, a.shape[0], n, k))
+    _, qn, sn, gn = f4.rand_marlin_weight_nvfp4_like(w16, 16)
+    gn = gn.view(1)
+    cases["nvfp4_f16"] = (torch.float16, 0.5, lambda a: ops.gptq_marlin_gemm(
+        a, None, qn, None, sn, gn, None, None, None, workspace, st.float4_e2m1f, a.shape[0], n, k))
+    _, qm, sm = f4.rand_marlin_weight_mxfp4_like(w16.bfloat16(), 32)
+    cases["mxfp4_bf16"] = (torch.bfloat16, 0.5, lambda a: ops.gptq_marlin_gemm(
+        a, None, qm, None, sm, None, None, None, None, workspace, st.float4_e2m1f, a.shape[0], n, k))
+    qh = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev)
+    sh = marlin_permute_scales(torch.rand(k // 64, n, dtype=torch.float16, device=dev) * 0.01, k, n, 64)
+    zh = marlin_permute_scales(torch.rand(k // 64, n, dtype=torch.float16, device=dev) * 8, k, n, 64)
+    cases["uint4_fp16_zero_points_g64"] = (torch.float16, 0.5, lambda a: ops.gptq_marlin_gemm(
+        a, None, qh, None, sh, None, zh, e, e, workspace, st.uint4, a.shape[0], n, k, is_zp_float=True))
+    out = {}
+    for label, (dt, bytes_per_weight, fn) in cases.items():
+        for m in (16, 4096):
+            a = torch.randn(m, k, device=dev).to(dt)
+            reps = 20 if m == 16 else 4
+            sec = time_graph([lambda: fn(a)] * reps, reps=5, warmup=1) / reps
+            out[f"{label}_M{m}"] = {"us": sec * 1e6, "TFLOPs": 2.0 * m * n * k / sec / 1e12,
+                                    "weight_GBps": k * n * bytes_per_weight / sec / 1e9}
+            print(f"[detail] gate_up {label} M={m}: {sec * 1e6:.1f} us, {2.0 * m * n * k / sec / 1e12:.0f} TFLOP/s, "
+                  f"{k * n * bytes_per_weight / sec / 1e9:.0f} GB/s of weights", file=sys.stderr, flush=True)
+    return out
+
+
 def _cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -476,6 +519,8 @@ def main():
         detail["mixtral_moe_fp16_gptq"] = bench_moe(ops, scalar_types.uint4b8, dev)
         torch.cuda.empty_cache()
         detail["repack"] = bench_repack(ops, dev)
+        torch.cuda.empty_cache()
+        detail["other_weight_types_gate_up_warm"] = bench_other_types(ops, dev, workspace)
         result["detail"] = detail
         result["summary"] = {
             "decode_fp16_gptq_us": {k: round(v["us"], 2) for k, v in detail["decode_fp16_gptq"].items()},
