@@ -104,6 +104,23 @@ def test_prefill_tiles(ops, dev, workspace):
     assert int(workspace.abs().sum()) == 0
 
 
+def test_64_row_tiles_with_split_k(ops, dev, workspace):
+    """136 tiles of 64 x 512: the 64-row kernel splits K in two and a second kernel adds the partial tiles."""
+    size_m, size_k, size_n = 512, 2048, 8704
+    _, _, _, mq, ms, mz = make_hqq(size_k, size_n, 14)
+    w = gr.dequant_marlin_float_zp(mq, ms, mz, size_k, size_n)
+    a = torch.randn(size_m, size_k, generator=torch.Generator().manual_seed(2)).half()
+    out = run(ops, a.to(dev), mq, ms, mz, workspace, size_n, size_k).cpu()
+    m = gr.error_metrics(out, gr.gemm_ref(a, w))
+    assert m["max_rel"] <= 2e-2 and m["mean_rel"] < 0.04, m
+    rows = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(5))
+    hot = torch.zeros(size_m, size_k, dtype=torch.float16)
+    hot[torch.arange(size_m), rows] = 1.0
+    out = run(ops, hot.to(dev), mq, ms, mz, workspace, size_n, size_k)
+    assert torch.equal(out.cpu(), w[rows])
+    assert int(workspace.abs().sum()) == 0
+
+
 def test_argument_errors(ops, dev, workspace):
     import vllm_amd.scalar_type as vst
     size_k, size_n = 256, 128

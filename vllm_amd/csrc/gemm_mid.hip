@@ -36,8 +36,10 @@ constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_B
 // k-steps); NVFP4's per-expert global scale is applied to the accumulator.
 // BITS = 8: uint8b128 or (FP8) float8_e4m3fn weights in the 8-bit Marlin layout; their stages hold twice the weight
 // registers, which still fits the two-workgroups-per-compute-unit budget (the grouped variants spill 2-9 registers).
-template <int DT, bool ZP, bool CHANNEL, bool MOE, int FP4 = 0, int BITS = 4, bool FP8 = false>
+// ZPF: uint4 weights with fp16 zero points laid out like the scales (HQQ; dense only).
+template <int DT, bool ZP, bool CHANNEL, bool MOE, int FP4 = 0, int BITS = 4, bool FP8 = false, bool ZPF = false>
 __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
+  static_assert(!ZPF || (DT == DT_F16 && !ZP && !CHANNEL && !MOE && BITS == 4 && FP4 == 0), "float zero points: fp16 uint4 grouped, dense");
   static_assert(FP4 == 0 || (!ZP && !CHANNEL && BITS == 4), "fp4 weights: grouped scale records, no zero points");
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights have no zero points");
   static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
@@ -102,6 +104,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const int64_t s_row = p.N >> 3;
   const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
+  const u32x4* zfp = ZPF ? (const u32x4*)Zp + nt * 8 + c : nullptr;  // fp16 zero points: indexed like the scales
 
   // ---- activation staging: thread t loads piece (t & 7) of tile rows (t >> 3) + 32 i, i = 0..1
   // (rows without a source read row 0 of A; their results are never stored)
@@ -145,6 +148,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   struct Stage {
     u32x4 b0, b1, sc;
     u32x4 b0h, b1h;  // 8-bit weights only: the thread's words 2, 3
+    u32x4 zf;        // float zero points only
     uint32_t zq;
   };
   Stage st[MD_D];
@@ -155,6 +159,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
     if (ZP) s.zq = zp[(int64_t)gi * s_row];
     if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
+    if (ZPF) s.zf = zfp[(int64_t)gi * s_row];
     s.b0 = bp[(int64_t)(2 * ks) * b_row];
     s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
     if constexpr (BITS == 8) {
@@ -208,7 +213,10 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   store_a(0);
   // B operands of two Marlin words: the one whose MFMAs are being issued and the one being dequantised
   u32x4 ob[2][2];
-  if constexpr (FP4 != 0) {
+  if constexpr (ZPF) {
+    dequant_pair_zpf(st[0].b0[0], st[0].b1[0], st[0].sc[0], as_u32(as_h2(st[0].zf[0]) * as_h2(st[0].sc[0])), ob[0][0],
+                     ob[0][1]);
+  } else if constexpr (FP4 != 0) {
     const Fp4Scales fs = fp4_scales(st[0], 0);
     dequant_pair_fp4<DT>(st[0].b0[0], st[0].b1[0], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][0], ob[0][1]);
   } else if constexpr (FP8) {
@@ -237,12 +245,16 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       const Stage& src = w == 3 ? nxt : cur;
       const ColConst<DT> cc = col_const(src, wn);
       const Fp4Scales fs = fp4_scales(src, wn);
+      uint32_t zs = 0;
+      if constexpr (ZPF) zs = as_u32(as_h2(src.zf[wn]) * as_h2(src.sc[wn]));
       const uint32_t xa = src.b0[wn], xb = src.b1[wn];
       auto step = [&](auto j_tag) {
         constexpr int J = decltype(j_tag)::value;
         mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
         uint32_t r;
-        if constexpr (FP4 != 0)
+        if constexpr (ZPF)
+          r = dequant_piece_zpf<J>(xa, xb, src.sc[wn], zs);
+        else if constexpr (FP4 != 0)
           r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
         else if constexpr (BITS == 8)
           r = dequant_piece8<DT, UNIT, FP8, J>(word8(src, wn, (J & 3) >> 1, 0), word8(src, wn, (J & 3) >> 1, 1),
@@ -462,7 +474,11 @@ int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   const bool moe = (a->flags & W4A16_F_MOE) != 0;
   mid_fn fn, red;
-  if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
+  if (a->flags & W4A16_F_ZP_FLOAT) {
+    if (a->dtype != DT_F16 || channel || moe) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    fn = mid_kernel<DT_F16, false, false, false, 0, 4, false, true>;
+    red = pick_reduce<DT_F16, false>(false);
+  } else if (a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3) {
     if (zp) return fail(W4A16_EINVAL, "unsupported kernel variant");
     const bool fp8 = a->wtype == W4A16_WTYPE_FE4M3;
     if (a->dtype == DT_F16) {
