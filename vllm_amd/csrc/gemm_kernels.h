@@ -153,6 +153,9 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
 // otherwise assigns different registers to an MFMA's source and destination accumulator and fills the loop
 // with v_accvgpr moves (more of them than dequantisation instructions).  Source C == destination is the form
 // the matrix pipe forwards without extra wait states; results are only read again after the main loop.
+// The statement is opaque to the compiler's hazard logic: an operand register must not be written by a VALU
+// instruction in the two wait states before it (callers dequantise operands several MFMAs ahead; a compiler-output
+// test checks the distance).
 template <int DT>
 __device__ __forceinline__ void mfma_inplace(f32x4& acc, const u32x4& a, const u32x4& b) {
   if constexpr (DT == DT_F16)
