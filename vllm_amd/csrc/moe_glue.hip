@@ -67,15 +67,25 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(
     int pos = off[e];
     const int end = off[e + 1];
     if (pos == end) continue;
-    for (int base = 0; base < numel; base += 64) {
-      const int i = base + lane;
-      const bool hit = i < numel && topk_ids[i] == e;
-      const unsigned long long m = __ballot(hit);
-      if (hit) {
-        const int rank = __popcll(m & ((1ull << lane) - 1ull));
-        if (pos + rank < sorted_len) sorted_ids[pos + rank] = i;
+    // four independent loads per round trip (the loop is latency-bound: 64 ids per wavefront and load otherwise)
+    for (int base = 0; base < numel; base += 256) {
+      int id[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = base + 64 * u + lane;
+        id[u] = i < numel ? topk_ids[i] : -1;
       }
-      pos += __popcll(m);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = base + 64 * u + lane;
+        const bool hit = id[u] == e;  // (e >= 0: padding ids never match)
+        const unsigned long long m = __ballot(hit);
+        if (hit) {
+          const int rank = __popcll(m & ((1ull << lane) - 1ull));
+          if (pos + rank < sorted_len) sorted_ids[pos + rank] = i;
+        }
+        pos += __popcll(m);
+      }
     }
     for (int i = pos + lane; i < end && i < sorted_len; i += 64) sorted_ids[i] = numel;
   }
