@@ -344,3 +344,24 @@ def test_split_k_with_short_workspaces(ops, dev, ws_len):
     big = torch.zeros(4096, dtype=torch.int32, device=dev)
     assert torch.equal(out, run_gemm(ops, layer, a, dev, big))
     assert torch.equal(out, run_gemm(ops, layer, a, dev, ws))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode,group", [("gptq", 128), ("gptq", -1), ("awq", 64), ("gptq_act_order", 128)])
+@pytest.mark.parametrize("size_m", [65, 100, 128])
+def test_two_row_tiles_of_256_columns(ops, dev, workspace, dtype, mode, group, size_m):
+    """65..128 rows and N wide enough that two row tiles of 64 x 256 give most compute units a workgroup: the kernel with
+    the in-workgroup K split.  N = 25664 leaves a partial 256-column tile; one-hot rows must be bit-exact."""
+    size_k, size_n = 1024, 25664
+    print(f"kq dtype={dtype} {mode} g={group} m={size_m}", flush=True)
+    layer = make_layer(size_k, size_n, group, dtype, has_zp=(mode == "awq"), act_order=(mode == "gptq_act_order"),
+                       seed=size_m)
+    a = _a(size_m, size_k, dtype, dev)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    ks = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(3))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), ks] = 1.0
+    out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    assert int(workspace.abs().sum()) == 0

@@ -1,7 +1,8 @@
-"""Compiler-output check for the kernels that issue MFMAs through inline assembly (gemm_fat.hip, gemm_mid.hip).
+"""Compiler-output check for the kernels that issue MFMAs through inline assembly (gemm_fat.hip, gemm_mid.hip,
+gemm_kq.hip).
 
 On gfx950 an MFMA that reads a VGPR fewer than two wait states after a VALU instruction wrote it sees the old value.
-The compiler keeps that distance for MFMAs it knows; an inline-assembly MFMA is opaque to it.  This test compiles the two
+The compiler keeps that distance for MFMAs it knows; an inline-assembly MFMA is opaque to it.  This test compiles the
 files to assembly (device pass only, no GPU needed) and fails if any MFMA source register is written by a VALU
 instruction with fewer than two wait states in between (every instruction counts one, `s_nop N` counts N + 1)."""
 import os
@@ -48,7 +49,7 @@ def _violations(path):
     return total, bad
 
 
-@pytest.mark.parametrize("src", ["gemm_fat.hip", "gemm_mid.hip"])
+@pytest.mark.parametrize("src", ["gemm_fat.hip", "gemm_mid.hip", "gemm_kq.hip"])
 def test_no_valu_write_right_before_an_asm_mfma(src):
     flags = [f for f in vbuild.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
     with tempfile.TemporaryDirectory() as tmp:
@@ -57,5 +58,5 @@ def test_no_valu_write_right_before_an_asm_mfma(src):
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         assert r.returncode == 0, r.stdout
         total, bad = _violations(out)
-    assert total >= 2048, total  # the kernels are there
+    assert total >= 1024, total  # the kernels are there (128 MFMAs per loop body and instantiation)
     assert not bad, bad[:5]

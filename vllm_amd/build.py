@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libw4a16_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
-SOURCES = ["c_api.hip", "repack.hip", "gemm.hip", "gemm_skinny.hip", "gemm_decode.hip", "gemm_fat.hip", "gemm_mid.hip", "moe_glue.hip"]
+SOURCES = ["c_api.hip", "repack.hip", "gemm.hip", "gemm_skinny.hip", "gemm_decode.hip", "gemm_fat.hip", "gemm_mid.hip", "gemm_kq.hip", "moe_glue.hip"]
 
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIPCC_FLAGS = [

@@ -165,7 +165,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     prefer_mid = mid_units < 0.95 * fat_units;
   }
   if (!moe && fat_ok && pow2_group && a->size_m >= 128 && !prefer_mid && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
-      pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3) {
+      pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3 && forced_kind != 5) {
     pl.kind = 2;
     pl.tn = 512;
     pl.mb = 8;
@@ -190,6 +190,35 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
         pl.tail_strips = (int)strips;
     }
     return 0;
+  }
+
+  // 64-row tiles of 256 columns with the K range cut in four inside the workgroup (one workgroup per compute unit).
+  {
+    const bool kq_shape = !moe && !general_only && pow2_group && pl.gm != GM_GIDX && a->size_k % 512 == 0 && a->size_m > 32;
+    // measured against the alternatives (16-row tiles, general kernel): ahead by 15-18 % at 65..128 rows when the two
+    // row tiles alone give at least 3/4 of the compute units a workgroup (gate_up: 45.6 / 48.5 us at 96 / 128 rows
+    // against 54 / 58), behind everywhere else
+    const int64_t kq_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 256);
+    const bool kq_pays = a->size_m > 64 && a->size_m <= 128 && kq_tiles >= cus * 3 / 4 && kq_tiles <= cus;
+    if (kq_shape && (forced_kind == 5 || (forced_kind < 0 && kq_pays))) {
+      pl.kind = 5;
+      pl.tn = 256;
+      pl.mb = 4;
+      pl.bm = 64;
+      pl.mtiles = (int)ceil_div(a->size_m, 64);
+      pl.ncp = (int)ceil_div(a->size_n, 256);
+      const int64_t tiles = (int64_t)pl.mtiles * pl.ncp;
+      W4A16_CHECK(tiles < (1LL << 31) / 64, "too many tiles");
+      pl.tiles = (int)tiles;
+      pl.splits = 1;
+      pl.kps = pl.total_ksteps;
+      pl.xcd_map = 0;
+      pl.ctmp_bytes = 0;
+      if (debug_plan)
+        fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=5 tiles=%d splits=%d kps=%d\n", (long long)a->size_m,
+                (long long)a->size_n, (long long)a->size_k, pl.tiles, pl.splits, pl.kps);
+      return 0;
+    }
   }
 
   // 64-row kernel: MoE blocks of 64 slots, and dense problems with too few rows or tiles for the prefill kernel.
@@ -363,5 +392,6 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
     return launch_mid(&b, tail, (hipStream_t)stream);
   }
   if (pl.kind == 3) return launch_mid(&b, pl, (hipStream_t)stream);
+  if (pl.kind == 5) return launch_kq(&b, pl, (hipStream_t)stream);
   return pl.kind == 1 ? launch_decode(&b, pl, (hipStream_t)stream) : launch_skinny(&b, pl, (hipStream_t)stream);
 }

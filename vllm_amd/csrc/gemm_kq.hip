@@ -1,0 +1,305 @@
+// W4A16 GEMM for gfx950 with 64-row tiles and an in-workgroup K split: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias),
+// dense, for 65..128 rows and wide N, where the 64 x 512 tiles of the 64-row kernel are too few to fill the chip
+// (the reference's small-batch thread configurations, csrc/quantization/gptq_marlin/gptq_marlin.cu:120-170).
+//
+//   workgroup tile 64 rows x 256 columns, 8 wavefronts = 2 column pairs x 4 K-quarters: every wavefront owns
+//   64 rows x 128 columns (32 v_mfma_f32_16x16x32 per k-step, 128 fp32 accumulators in AGPRs) over a quarter of the
+//   K range, two wavefronts per SIMD.
+//   weights      streamed global -> registers per wavefront and dequantised one operand register per MFMA, exactly as
+//                in the 64-row kernel (B operand = the reference's half(q - z) * half(s)).
+//   activations  each K-quarter stages its own 64 rows x 64 K chunk into LDS in MFMA fragment order (its two
+//                wavefronts share it), double buffered; one workgroup barrier per two k-steps.
+//   epilogue     the four quarters' partial tiles are added through LDS, one 16-row block at a time.
+//   No split across workgroups: the planner only picks this kernel when its tiles about fill the chip (with too few
+//   tiles the partial tiles in HBM and the second launch cost more than the 16-row tiles they would replace).
+// Compared with 16-row tiles (which re-read and re-convert the weight strip once per 16 rows) every weight is fetched
+// and dequantised once per 64 rows; compared with the 64 x 512 tile there are 2 x 4 times as many independent streams.
+// Requirements (host-checked): K % 512 == 0 (every quarter runs whole ring periods of 4 k-steps), scales grouped (a
+// power-of-two number of k-steps) or channelwise, no per-row g_idx, A's columns already in weight order.
+#include <type_traits>
+
+#include "gemm_kernels.h"
+
+namespace w4a16 {
+
+constexpr int KQ_MB = 4;     // m-blocks per tile
+constexpr int KQ_BM = 64;    // rows per tile
+constexpr int KQ_TN = 256;   // columns per tile
+constexpr int KQ_Q = 4;      // K-quarters
+constexpr int KQ_D = 4;      // weight k-steps in flight per wavefront
+constexpr int KQ_ABUF = 2 * KQ_MB * 64 * 16;                 // one A buffer of one quarter: 2 k-steps x 4 m-blocks x 64 lanes x 16 B
+constexpr int KQ_SLABS = 8 * 16 * RED_RS * 4;                // eight wavefront slabs of the epilogue
+constexpr int KQ_STAGE = KQ_Q * 2 * KQ_ABUF;
+constexpr int KQ_SMEM = (KQ_STAGE > KQ_SLABS ? KQ_STAGE : KQ_SLABS) + KQ_BM * 4;  // + C row of each tile row
+
+template <int DT, bool ZP, bool CHANNEL>
+__global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
+  constexpr bool UNIT = CHANNEL;
+  extern __shared__ __align__(16) unsigned char smem[];
+  int* s_crow = (int*)(smem + KQ_SMEM - KQ_BM * 4);
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wn = wv & 1, q = wv >> 1;  // column pair inside the tile, K-quarter
+  const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
+
+  // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
+  const int mtiles = (p.M + KQ_BM - 1) / KQ_BM;
+  const int mt = blockIdx.x % mtiles;
+  const int strip = blockIdx.x / mtiles;
+  const int cp = strip * 2 + wn;               // column pair of this wavefront
+  const bool wave_on = cp * 128 < p.N;         // N not a multiple of 256: the trailing wavefronts only help staging
+  const int row0 = mt * KQ_BM;
+
+  const uint32_t* Bq = p.B;
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint32_t* Zp = p.Z;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  // which A row feeds tile row r and which C row receives it (-1: none)
+  auto tile_row_ids = [&](int r, int& src, int& dst) {
+    src = dst = -1;
+    if (row0 + r < p.M) src = dst = row0 + r;
+  };
+  if (t < KQ_BM) {
+    int src, dst;
+    tile_row_ids(t, src, dst);
+    s_crow[t] = dst;
+  }
+
+  // ---- weights of this wavefront
+  const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
+  const int64_t b_row = p.N >> 1;
+  const u32x4* bp = (const u32x4*)Bq + nt * 32 + (4 * c + g);
+  const int64_t s_row = p.N >> 3;
+  const u32x4* sp = (const u32x4*)Sc + nt * 8 + c;
+  const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
+
+  // ---- this quarter's k-steps: [ks_b, ks_e), a multiple of 4 long
+  const int per_q = p.total_ksteps / KQ_Q;  // host: a multiple of 4
+  const int ks_b = q * per_q, ks_e = ks_b + per_q;
+
+  // ---- activation staging: the quarter's 128 threads; thread tq loads piece (tq & 7) of tile rows (tq >> 3) + 16 i
+  // (rows without a source read row 0 of A; their results are never stored)
+  const int tq = wn * 64 + lane;
+  const int piece = tq & 7;
+  const uint16_t* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int src, dst;
+    tile_row_ids((tq >> 3) + 16 * i, src, dst);
+    arow[i] = (const uint16_t*)p.A + (int64_t)(src < 0 ? 0 : src) * p.lda + piece * 8;
+  }
+  // LDS A layout per quarter: [buffer][k-step 2][m-block 4][lane 64][4 dwords]; the 16 bytes of (row, piece) are the
+  // K pairs 8*pp + 2j (pp = piece & 3), which belong to lane (j*16 + row%16), dword pp, of k-step piece >> 2.
+  uint32_t* lds = (uint32_t*)smem + q * (2 * KQ_ABUF / 4);
+  int a_wr[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tq >> 3) + 16 * i;
+    a_wr[i] = (((piece >> 2) * KQ_MB + (r >> 4)) * 64 + (r & 15)) * 4 + (piece & 3);
+  }
+  u32x4 areg[4];
+  // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
+  //  keeps the main loop free of branches)
+  auto load_a = [&](int chunk) {  // chunk: relative to ks_b
+    chunk = min(ks_b / 2 + chunk, ks_e / 2 - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
+  };
+  auto store_a = [&](int buf) {
+    uint32_t* dst = lds + buf * (KQ_ABUF / 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[a_wr[i] + j * 64] = areg[i][j];
+    }
+  };
+
+  struct Stage {
+    u32x4 b0, b1, sc;
+    uint32_t zq;
+  };
+  Stage st[KQ_D];
+  auto issue = [&](Stage& s, int ks) {  // ks: relative to ks_b
+    ks = min(ks_b + ks, ks_e - 1);
+    int gi = 0;
+    if (!CHANNEL) gi = ks >> p.group_shift;
+    if (!CHANNEL) s.sc = sp[(int64_t)gi * s_row];
+    if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    s.b0 = bp[(int64_t)(2 * ks) * b_row];
+    s.b1 = bp[(int64_t)(2 * ks + 1) * b_row];
+  };
+  auto col_const = [&](const Stage& s, int w) {
+    uint32_t z0 = 8, z1 = 8;
+    if (ZP) {
+      z0 = (s.zq >> (4 * w)) & 0xf;
+      z1 = (s.zq >> (4 * w + 16)) & 0xf;
+    }
+    return make_col_const<DT, UNIT>(CHANNEL ? 0u : s.sc[w], z0, z1);
+  };
+
+  f32x4 acc[KQ_MB][4][2];
+#pragma unroll
+  for (int mb = 0; mb < KQ_MB; ++mb)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      acc[mb][w][0] = f32x4{0, 0, 0, 0};
+      acc[mb][w][1] = f32x4{0, 0, 0, 0};
+    }
+
+  const int nchunks = per_q / 2;  // even
+
+  // ---- prologue
+  load_a(0);
+#pragma unroll
+  for (int j = 0; j < KQ_D; ++j) issue(st[j], j);
+  store_a(0);
+  // B operands of two Marlin words: the one whose MFMAs are being issued and the one being dequantised
+  u32x4 ob[2][2];
+  {
+    const ColConst<DT> cc = col_const(st[0], 0);
+    dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], cc, ob[0][0], ob[0][1]);
+  }
+  __syncthreads();
+
+  // One k-step: per Marlin word w, 8 MFMAs on ob[w & 1]; after each MFMA one register of the following word's
+  // operands (word w + 1 of this k-step, or word 0 of the next k-step `nxt`) is dequantised into ob[(w + 1) & 1].
+  // The scheduling barriers keep the compiler from regrouping this into MFMA-only and VALU-only blocks.
+  auto kstep = [&](int buf, int kk, const Stage& cur, const Stage& nxt) {
+    const u32x4* abase = (const u32x4*)(lds + buf * (KQ_ABUF / 4)) + (kk * KQ_MB) * 64 + lane;
+    u32x4 af[KQ_MB];
+#pragma unroll
+    for (int mb = 0; mb < KQ_MB; ++mb) af[mb] = abase[mb * 64];
+    auto word = [&](auto w_tag) {
+      constexpr int w = decltype(w_tag)::value;
+      constexpr int wn2 = (w + 1) & 3;
+      const Stage& src = w == 3 ? nxt : cur;
+      const ColConst<DT> cc = col_const(src, wn2);
+      const uint32_t xa = src.b0[wn2], xb = src.b1[wn2];
+      auto step = [&](auto j_tag) {
+        constexpr int J = decltype(j_tag)::value;
+        mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
+        const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
+        if constexpr (J < 4)
+          ob[wn2 & 1][0][J] = r;
+        else
+          ob[wn2 & 1][1][J - 4] = r;
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      step(std::integral_constant<int, 0>{});
+      step(std::integral_constant<int, 1>{});
+      step(std::integral_constant<int, 2>{});
+      step(std::integral_constant<int, 3>{});
+      step(std::integral_constant<int, 4>{});
+      step(std::integral_constant<int, 5>{});
+      step(std::integral_constant<int, 6>{});
+      step(std::integral_constant<int, 7>{});
+    };
+    word(std::integral_constant<int, 0>{});
+    word(std::integral_constant<int, 1>{});
+    word(std::integral_constant<int, 2>{});
+    word(std::integral_constant<int, 3>{});
+  };
+
+  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration; all quarters run the same count
+#pragma unroll 1
+  for (int c0 = 0; c0 < nchunks; c0 += 2) {
+    const int ks0 = 2 * c0;
+    load_a(c0 + 1);
+    kstep(0, 0, st[0], st[1]);
+    issue(st[0], ks0 + 4);
+    kstep(0, 1, st[1], st[2]);
+    issue(st[1], ks0 + 5);
+    store_a(1);
+    __syncthreads();
+    load_a(c0 + 2);
+    kstep(1, 0, st[2], st[3]);
+    issue(st[2], ks0 + 6);
+    kstep(1, 1, st[3], st[0]);
+    issue(st[3], ks0 + 7);
+    store_a(0);
+    __syncthreads();
+  }
+
+  // ------------------------------------------------------------------------------ epilogue
+  // (the inline-asm MFMAs are opaque to the compiler's hazard logic: let the matrix pipe drain before the
+  //  accumulators are read)
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // per m-block: every wavefront writes its 16 x 128 partial to its slab [16 rows][RED_RS]; after a barrier the
+  // wavefront of quarter q adds the four quarters' slabs of its column pair for rows 4q .. 4q+3 and finishes them.
+  // (the last barrier of the loop separates the slabs from the A buffers they overlay)
+  float* slabs = (float*)smem;
+  float* mine = slabs + wv * (16 * RED_RS);
+  const int fc4 = (lane & 31) * 4;
+  const int fpos = fc4 + (fc4 >= 64 ? 8 : 0);
+  const int ncol = cp * 128 + fc4;
+  const bool fcol_ok = wave_on && ncol < p.N;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  if (fcol_ok) {
+    const int base = ncol & ~31, cl = ncol & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  }
+#pragma unroll
+  for (int mb = 0; mb < KQ_MB; ++mb) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mine[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r16 = 4 * q + (lane >> 5) + 2 * i;
+      const int crow = s_crow[mb * 16 + r16];
+      f32x4 v = {0, 0, 0, 0};
+#pragma unroll
+      for (int qq = 0; qq < KQ_Q; ++qq) v += *(const f32x4*)(slabs + (qq * 2 + wn) * (16 * RED_RS) + r16 * RED_RS + fpos);
+      if (fcol_ok && crow >= 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+        u32x2 o;
+        if constexpr (DT == DT_F16)
+          o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+        else
+          o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+        *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+typedef void (*kq_fn)(const KParams);
+
+template <int DT>
+static kq_fn pick_kq(bool zp, bool channel) {
+  if (zp) return channel ? kq_kernel<DT, true, true> : kq_kernel<DT, true, false>;
+  return channel ? kq_kernel<DT, false, true> : kq_kernel<DT, false, false>;
+}
+
+int launch_kq(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
+  const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
+  if ((a->wtype != W4A16_WTYPE_U4B8 && a->wtype != W4A16_WTYPE_U4) || (a->flags & (W4A16_F_ZP_FLOAT | W4A16_F_MOE)) ||
+      pl.gm == GM_GIDX || pl.use_perm || a->size_k % 512 != 0 || pl.splits != 1 || pl.tn != KQ_TN)
+    return fail(W4A16_EINVAL, "unsupported kernel variant");
+  const kq_fn fn = a->dtype == DT_F16 ? pick_kq<DT_F16>(zp, channel) : pick_kq<DT_BF16>(zp, channel);
+  KParams p = make_kparams(a, pl);
+  if (pl.tiles <= 0) return 0;
+  W4A16_HIP(allow_dynamic_lds((const void*)fn, KQ_SMEM));
+  hipLaunchKernelGGL(fn, dim3((unsigned)pl.tiles), dim3(512), KQ_SMEM, stream, p);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace w4a16

@@ -12,7 +12,8 @@ struct Plan {
   int mtiles, ncp, tiles;
   int total_ksteps, splits, kps;  // k-steps of 32 rows; K splits; k-steps per split
   int xcd_map;
-  int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel, 3: 64-row ("mid") kernel
+  int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel, 3: 64-row ("mid") kernel,
+             // 5: 64-row kernel with the in-workgroup K split (gemm_kq.hip)
   int tn;    // tile width in columns (128; the decode kernel also has 64)
   int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
   int tail_strips = 0; // prefill plan: trailing 512-column strips handed to the 64-row kernel (0 = none)
@@ -24,5 +25,6 @@ int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_fat(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
+int launch_kq(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 
 }  // namespace w4a16
