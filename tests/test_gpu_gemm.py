@@ -365,3 +365,19 @@ def test_two_row_tiles_of_256_columns(ops, dev, workspace, dtype, mode, group, s
     out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
     assert torch.equal(out.cpu(), layer.w_ref[ks])
     assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype,mode,group", [(torch.float16, "gptq", 128), (torch.bfloat16, "awq", 128)])
+def test_one_row_tile_of_256_columns(ops, dev, workspace, dtype, mode, group):
+    """33..64 rows with N so wide (193 tiles of 256 columns) that one row tile fills the chip: same kernel as above."""
+    size_m, size_k, size_n = 40, 512, 49216
+    layer = make_layer(size_k, size_n, group, dtype, has_zp=(mode == "awq"), seed=77)
+    a = _a(size_m, size_k, dtype, dev)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    check_close(out, a, layer)
+    ks = torch.randint(0, size_k, (size_m,), generator=torch.Generator().manual_seed(3))
+    hot = torch.zeros(size_m, size_k, dtype=dtype)
+    hot[torch.arange(size_m), ks] = 1.0
+    out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    assert int(workspace.abs().sum()) == 0

@@ -195,11 +195,11 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // 64-row tiles of 256 columns with the K range cut in four inside the workgroup (one workgroup per compute unit).
   {
     const bool kq_shape = !moe && !general_only && pow2_group && pl.gm != GM_GIDX && a->size_k % 512 == 0 && a->size_m > 32;
-    // measured against the alternatives (16-row tiles, general kernel): ahead by 15-18 % at 65..128 rows when the two
-    // row tiles alone give at least 3/4 of the compute units a workgroup (gate_up: 45.6 / 48.5 us at 96 / 128 rows
-    // against 54 / 58), behind everywhere else
+    // measured against the alternatives (16-row tiles, general kernel): ahead by 13-25 % at 33..128 rows when its tiles
+    // give between 3/4 and all of the compute units a workgroup (4096 x 28672: 45 / 44 us at 96 / 128 rows against
+    // 54 / 58; 8192 x 57344: 75-82 us at 33-64 rows against 87-101), level at 1.75 rounds, behind with fewer tiles
     const int64_t kq_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 256);
-    const bool kq_pays = a->size_m > 64 && a->size_m <= 128 && kq_tiles >= cus * 3 / 4 && kq_tiles <= cus;
+    const bool kq_pays = a->size_m <= 128 && kq_tiles >= cus * 3 / 4 && kq_tiles <= cus;
     if (kq_shape && (forced_kind == 5 || (forced_kind < 0 && kq_pays))) {
       pl.kind = 5;
       pl.tn = 256;

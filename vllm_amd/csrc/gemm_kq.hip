@@ -1,5 +1,5 @@
 // W4A16 GEMM for gfx950 with 64-row tiles and an in-workgroup K split: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias),
-// dense, for 65..128 rows and wide N, where the 64 x 512 tiles of the 64-row kernel are too few to fill the chip
+// dense, for 33..128 rows and wide N, where the 64 x 512 tiles of the 64-row kernel are too few to fill the chip
 // (the reference's small-batch thread configurations, csrc/quantization/gptq_marlin/gptq_marlin.cu:120-170).
 //
 //   workgroup tile 64 rows x 256 columns, 8 wavefronts = 2 column pairs x 4 K-quarters: every wavefront owns
