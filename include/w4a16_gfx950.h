@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define W4A16_ABI_VERSION 2
+#define W4A16_ABI_VERSION 3
 
 enum {
   W4A16_OK = 0,
@@ -128,6 +128,18 @@ int64_t w4a16_gemm_scratch_bytes(const w4a16_gemm_args* args);
 
 /* Replaces torch.ops._C.gptq_marlin_gemm / torch.ops._moe_C.moe_wna16_marlin_gemm (see above). */
 int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream);
+
+/* The same GEMM for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, whose op allocates c_tmp and a_tmp itself
+ * (gptq_marlin.cu:751-763).  args->c_tmp, args->workspace and args->workspace_len are ignored: split-K partial
+ * tiles, the column-gathered copy of A (act-order) and the arrival counters live in a buffer of
+ * W4A16_STATIC_SCRATCH_BYTES inside the library's own device memory, one per GPU, held until the process ends.
+ * A problem that needs more scratch than that (w4a16_gemm_scratch_bytes says how much) fails with W4A16_EINVAL and a
+ * message; nothing is launched then.  The call allocates and frees nothing.  All calls on one GPU share that GPU's
+ * buffer: calls that overlap in time on one GPU (two streams, two host threads) race and must be serialised by the
+ * caller.  Inputs and the output are the caller's, as in w4a16_marlin_gemm, and results are identical to it. */
+#define W4A16_STATIC_SCRATCH_BYTES (64u << 20)
+int w4a16_marlin_gemm_static(const w4a16_gemm_args* args, void* stream);
 
 /* Replaces torch.ops._moe_C.moe_align_block_size
  * (csrc/moe/moe_align_sum_kernels.cu:275-346, schema csrc/moe/torch_bindings.cpp:17-23).

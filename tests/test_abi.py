@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert sorted(_lib.EXPORTS) == declared_functions()          # the ctypes table covers the header exactly
-    assert lib.w4a16_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.w4a16_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_args_struct_matches_header_layout():

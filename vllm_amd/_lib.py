@@ -10,9 +10,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libw4a16_gfx950.so")
 
 W4A16_OK = 0
+STATIC_SCRATCH_BYTES = 64 << 20  # W4A16_STATIC_SCRATCH_BYTES
 WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128, WTYPE_FE4M3, WTYPE_FE2M1 = 0, 1, 2, 3, 4
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 2  # W4A16_ABI_VERSION of include/w4a16_gfx950.h this mirror was written against
+ABI_VERSION = 3  # W4A16_ABI_VERSION of include/w4a16_gfx950.h this mirror was written against
 F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE, F_ZP_FLOAT = 1, 2, 4, 8, 16, 32
 
 c_void_p, c_i64, c_i32, c_u32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32
@@ -42,6 +43,7 @@ EXPORTS = {
     "w4a16_permute_cols": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
     "w4a16_gemm_scratch_bytes": (c_i64, [ctypes.POINTER(GemmArgs)]),
     "w4a16_marlin_gemm": (ctypes.c_int, [ctypes.POINTER(GemmArgs), c_void_p]),
+    "w4a16_marlin_gemm_static": (ctypes.c_int, [ctypes.POINTER(GemmArgs), c_void_p]),
     "w4a16_moe_align_block_size": (ctypes.c_int, [c_void_p, c_i64, c_i32, c_i32, c_void_p, c_i64, c_void_p,
                                                   c_i64, c_void_p, c_void_p]),
     "w4a16_moe_sum": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i32, c_i64, c_i32, c_void_p]),

@@ -3,7 +3,7 @@
 // csrc/moe/marlin_moe_wna16/ops.cu:691-993), launch planning, kernel dispatch.
 #include <stdlib.h>
 
-#include "gemm_plan.h"
+#include "gemm_kernels.h"
 
 namespace w4a16 {
 
@@ -359,15 +359,8 @@ extern "C" int64_t w4a16_gemm_scratch_bytes(const w4a16_gemm_args* args) {
   return ((pl.ctmp_bytes + 255) & ~255LL) + pl.atmp_bytes;
 }
 
-extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
-  if (int rc = validate(args)) return rc;
-  if (args->size_m == 0) return 0;
-  Plan pl;
-  if (int rc = make_plan(args, pl)) return rc;
-  if (pl.mtiles == 0) return 0;
-  if (pl.ctmp_bytes + pl.atmp_bytes > 0)
-    W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed",
-                (long long)(pl.ctmp_bytes + pl.atmp_bytes));
+// Launches the planned kernels; `args` already carries the scratch (c_tmp) and counter (workspace) pointers to use.
+static int run_planned(const w4a16_gemm_args* args, Plan& pl, void* stream) {
   w4a16_gemm_args b = *args;
   if (pl.atmp_bytes > 0) {
     void* a_tmp = (char*)args->c_tmp + ((pl.ctmp_bytes + 255) & ~255LL);
@@ -394,4 +387,77 @@ extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
   if (pl.kind == 3) return launch_mid(&b, pl, (hipStream_t)stream);
   if (pl.kind == 5) return launch_kq(&b, pl, (hipStream_t)stream);
   return pl.kind == 1 ? launch_decode(&b, pl, (hipStream_t)stream) : launch_skinny(&b, pl, (hipStream_t)stream);
+}
+
+extern "C" int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream) {
+  if (int rc = validate(args)) return rc;
+  if (args->size_m == 0) return 0;
+  Plan pl;
+  if (int rc = make_plan(args, pl)) return rc;
+  if (pl.mtiles == 0) return 0;
+  if (pl.ctmp_bytes + pl.atmp_bytes > 0)
+    W4A16_CHECK(args->c_tmp != nullptr, "c_tmp is null but %lld bytes are needed",
+                (long long)(pl.ctmp_bytes + pl.atmp_bytes));
+  return run_planned(args, pl, stream);
+}
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// Split-K partial tiles, the column-gathered copy of A (act-order) and the tiles' arrival counters live in one array
+// in the library's own device memory: W4A16_STATIC_SCRATCH_BYTES of data followed by STATIC_COUNTERS counters.
+// Every GPU the library runs on holds its own copy at its own address; host code only ever uses the address that
+// hipGetSymbolAddress returned for the current device.
+namespace w4a16 {
+constexpr int64_t STATIC_COUNTERS = 4096;
+static __device__ __align__(256) unsigned char scratch[W4A16_STATIC_SCRATCH_BYTES + STATIC_COUNTERS * 4];
+
+static int static_scratch(unsigned char** out) {
+  static std::mutex mu;
+  static unsigned char* ptrs[64] = {nullptr};
+  int dev = 0;
+  W4A16_HIP(hipGetDevice(&dev));
+  W4A16_CHECK(dev >= 0 && dev < 64, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    W4A16_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    W4A16_CHECK(p != nullptr, "hipGetSymbolAddress returned a null address for the static scratch");
+    ptrs[dev] = (unsigned char*)p;
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+
+__global__ void clear_counters_kernel(int32_t* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+}  // namespace w4a16
+
+extern "C" int w4a16_marlin_gemm_static(const w4a16_gemm_args* args, void* stream) {
+  if (int rc = validate(args)) return rc;
+  if (args->size_m == 0) return 0;
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  w4a16_gemm_args b = *args;
+  b.c_tmp = (float*)base;
+  b.workspace = (int32_t*)(base + W4A16_STATIC_SCRATCH_BYTES);
+  b.workspace_len = STATIC_COUNTERS;
+  Plan pl;
+  if (int rc = make_plan(&b, pl)) return rc;
+  if (pl.mtiles == 0) return 0;
+  const int64_t need = ((pl.ctmp_bytes + 255) & ~255LL) + pl.atmp_bytes;
+  W4A16_CHECK(need <= (int64_t)W4A16_STATIC_SCRATCH_BYTES,
+              "w4a16_marlin_gemm_static: this problem needs %lld bytes of scratch, the library's static buffer holds "
+              "%lld; use w4a16_marlin_gemm with a caller-owned c_tmp",
+              (long long)need, (long long)W4A16_STATIC_SCRATCH_BYTES);
+  if (pl.splits > 1 && (pl.kind == 0 || pl.kind == 1)) {
+    // arrival counters must start at zero; a fill kernel rather than a memset node, so that the call can be captured
+    const KParams kp = make_kparams(&b, pl);
+    const int n = pl.tiles * kp.lock_stride;
+    W4A16_CHECK(n <= STATIC_COUNTERS, "w4a16_marlin_gemm_static: %d arrival counters needed, %lld available", n,
+                (long long)STATIC_COUNTERS);
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, b.workspace, n);
+    W4A16_HIP(hipGetLastError());
+  }
+  return run_planned(&b, pl, stream);
 }
