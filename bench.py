@@ -44,54 +44,26 @@ def algorithmic_bytes(m, k, n, zp=False, act_order=False):
 
 
 # ------------------------------------------------------------------ synthetic layers (on the GPU)
-def _pack_rows_gpu(q):  # [K, N] int -> GPTQ int32 [K/8, N]
-    k, n = q.shape
-    f = q.to(torch.int64).reshape(k // 8, 8, n)
-    sh = (torch.arange(8, device=q.device, dtype=torch.int64) * 4).view(1, 8, 1)
-    w = (f << sh).sum(dim=1)
-    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32).contiguous()
-
-
-def _pack_cols_awq_gpu(q):  # [K, N] int -> AWQ int32 [K, N/8]
-    k, n = q.shape
-    order = torch.tensor([0, 2, 4, 6, 1, 3, 5, 7], device=q.device)
-    f = q.to(torch.int64).reshape(k, n // 8, 8)[:, :, order]
-    sh = (torch.arange(8, device=q.device, dtype=torch.int64) * 4).view(1, 1, 8)
-    w = (f << sh).sum(dim=2)
-    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32).contiguous()
+def _weights(k, n, dtype, dev, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(k, n, generator=g) * 0.02).to(dtype).to(dev)
 
 
 def make_gptq_layer(ops, k, n, dtype, dev, seed):
     """N(0, 0.02) weights, symmetric uint4b8 RTN, s = absmax/7 per (group, column)."""
-    from vllm_amd.marlin_utils import marlin_permute_scales
-    g = torch.Generator(device="cpu").manual_seed(seed)
-    w = (torch.randn(k, n, generator=g) * 0.02).to(dtype).to(dev)
-    wg = w.float().reshape(k // GROUP, GROUP, n)
-    s = (wg.abs().amax(dim=1, keepdim=True) / 7).clamp(min=1e-5).to(dtype)
-    q = torch.clamp(torch.round(wg / s.float()), -8, 7).to(torch.int32)
-    w_deq = (q.to(dtype) * s).reshape(k, n)
-    packed = _pack_rows_gpu((q + 8).reshape(k, n))
-    mq = ops.gptq_marlin_repack(packed, torch.empty(0, dtype=torch.int32, device=dev), k, n, 4)
-    ms = marlin_permute_scales(s.reshape(k // GROUP, n), k, n, GROUP)
-    return {"k": k, "n": n, "q": mq, "s": ms, "zp": torch.empty(0, dtype=torch.int32, device=dev), "w_deq": w_deq,
-            "packed": packed, "scales": s.reshape(k // GROUP, n)}
+    from vllm_amd.marlin_utils_test import marlin_quantize
+    from vllm_amd.scalar_type import scalar_types
+    w_ref, mq, ms, _, _, _ = marlin_quantize(_weights(k, n, dtype, dev, seed), scalar_types.uint4b8, GROUP, False,
+                                             rule="absmax")
+    return {"k": k, "n": n, "q": mq, "s": ms, "zp": torch.empty(0, dtype=torch.int32, device=dev), "w_deq": w_ref}
 
 
 def make_awq_layer(ops, k, n, dtype, dev, seed):
     """N(0, 0.02) weights, asymmetric uint4 RTN from per-group min/max, uint4 zero points."""
-    from vllm_amd.marlin_utils import awq_to_marlin_zero_points, marlin_permute_scales
-    g = torch.Generator(device="cpu").manual_seed(seed)
-    w = (torch.randn(k, n, generator=g) * 0.02).to(dtype).to(dev)
-    wg = w.float().reshape(k // GROUP, GROUP, n)
-    hi, lo = wg.amax(dim=1, keepdim=True), wg.amin(dim=1, keepdim=True)
-    s = ((hi - lo) / 15).clamp(min=1e-5).to(dtype)
-    z = torch.clamp(torch.round(-lo / s.float()), 0, 15).to(torch.int32)
-    q = torch.clamp(torch.round(wg / s.float()).to(torch.int32) + z, 0, 15)
-    w_deq = ((q - z).to(dtype) * s).reshape(k, n)
-    mq = ops.awq_marlin_repack(_pack_cols_awq_gpu(q.reshape(k, n)), k, n, 4)
-    ms = marlin_permute_scales(s.reshape(k // GROUP, n), k, n, GROUP)
-    mz = awq_to_marlin_zero_points(_pack_cols_awq_gpu(z.reshape(k // GROUP, n)), k // GROUP, n, 4)
-    return {"k": k, "n": n, "q": mq, "s": ms, "zp": mz, "w_deq": w_deq}
+    from vllm_amd.marlin_utils_test import awq_marlin_quantize
+    from vllm_amd.scalar_type import scalar_types
+    w_ref, mq, ms, mz = awq_marlin_quantize(_weights(k, n, dtype, dev, seed), scalar_types.uint4, GROUP, rule="absmax")
+    return {"k": k, "n": n, "q": mq, "s": ms, "zp": mz, "w_deq": w_ref}
 
 
 def clone_weights(layer, seed):
@@ -168,19 +140,13 @@ def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=4
 def make_gptq_actorder_layer(ops, k, n, dtype, dev, seed):
     """GPTQ desc_act layer: rows arrive in a seeded random order, g_idx[i] = group of arriving row i
     (as the reference's permute_rows, quant_utils.py:346-373); weights are repacked in group-sorted order."""
-    base = make_gptq_layer(ops, k, n, dtype, dev, seed)
-    g = torch.Generator(device="cpu").manual_seed(seed + 7)
-    perm = torch.randperm(k, generator=g).to(dev)
-    g_idx = (perm // GROUP).to(torch.int32)
-    order = torch.argsort(g_idx, stable=True).to(torch.int32)
-    packed_arrival = _pack_rows_gpu(_unpack_rows_gpu(base["packed"])[perm])
-    mq = ops.gptq_marlin_repack(packed_arrival, order, k, n, 4)
-    return {**base, "q": mq, "g_idx": g_idx[order.long()].contiguous(), "perm": order, "w_deq": base["w_deq"][perm]}
-
-
-def _unpack_rows_gpu(p):  # GPTQ int32 [K/8, N] -> [K, N]
-    sh = (torch.arange(8, device=p.device, dtype=torch.int64) * 4).view(1, 8, 1)
-    return (((p.to(torch.int64) & 0xFFFFFFFF).unsqueeze(1) >> sh) & 0xF).reshape(-1, p.shape[1]).to(torch.int32)
+    from vllm_amd.marlin_utils_test import marlin_quantize
+    from vllm_amd.scalar_type import scalar_types
+    perm = torch.randperm(k, generator=torch.Generator(device="cpu").manual_seed(seed + 7))
+    w_ref, mq, ms, g_idx, sort_idx, _ = marlin_quantize(_weights(k, n, dtype, dev, seed), scalar_types.uint4b8, GROUP,
+                                                        True, perm, rule="absmax")
+    return {"k": k, "n": n, "q": mq, "s": ms, "zp": torch.empty(0, dtype=torch.int32, device=dev), "w_deq": w_ref,
+            "g_idx": g_idx, "perm": sort_idx}
 
 
 def bench_repack(ops, dev):

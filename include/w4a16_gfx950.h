@@ -70,6 +70,23 @@ int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t s
 int w4a16_permute_cols(const void* a, const int32_t* perm, void* out, int64_t size_m,
                        int64_t size_k, int64_t lda, void* stream);
 
+/* Replaces the load-time helper marlin_permute_scales / marlin_permute_bias
+ * (vllm/model_executor/layers/quantization/utils/marlin_utils.py:278-305), which the reference runs as torch index
+ * ops.  s, out: 16-bit elements [num_rows, size_n], size_n a multiple of 64.  grouped != 0: the 8 x 8 transpose inside
+ * every 64-column chunk (group scales); grouped == 0: the "single" permutation inside every 32-column chunk
+ * (channel-wise scales, bias). */
+int w4a16_marlin_permute_scales(const void* s, void* out, int64_t num_rows, int64_t size_n, int grouped,
+                                void* stream);
+
+/* Replaces the load-time helpers marlin_zero_points / awq_to_marlin_zero_points (marlin_utils.py:326-370), which the
+ * reference runs in numpy on the host (quant_utils.py:548-602).  out: int32 [num_groups, size_n/8], Marlin packing.
+ * format 0: zp int32 [num_groups, size_n/8], nibble j of word c = column 8c + j (what
+ *           unpack_cols(x.t()) of MarlinLinearKernel.process_weights_after_loading starts from, marlin.py:115-133);
+ * format 1: the same shape in AWQ packing (column 8c + j in nibble {0,4,1,5,2,6,3,7}[j]);
+ * format 2: unpacked int32 [num_groups, size_n] (the argument of marlin_zero_points). */
+int w4a16_marlin_zero_points(const uint32_t* zp, uint32_t* out, int64_t num_groups, int64_t size_n, int format,
+                             void* stream);
+
 /* Operands of one W4A16 GEMM  C[M,N] = A[M,K] * dequant(Bq)[K,N] (+ bias).
  * Mirrors the tensor arguments of torch.ops._C.gptq_marlin_gemm
  * (csrc/quantization/gptq_marlin/gptq_marlin.cu:674-959, schema csrc/torch_bindings.cpp:316-323)

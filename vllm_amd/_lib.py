@@ -41,6 +41,8 @@ EXPORTS = {
     "w4a16_gptq_marlin_repack": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, ctypes.c_int, c_void_p]),
     "w4a16_awq_marlin_repack": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i64, ctypes.c_int, c_void_p]),
     "w4a16_permute_cols": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
+    "w4a16_marlin_permute_scales": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i64, ctypes.c_int, c_void_p]),
+    "w4a16_marlin_zero_points": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i64, ctypes.c_int, c_void_p]),
     "w4a16_gemm_scratch_bytes": (c_i64, [ctypes.POINTER(GemmArgs)]),
     "w4a16_marlin_gemm": (ctypes.c_int, [ctypes.POINTER(GemmArgs), c_void_p]),
     "w4a16_marlin_gemm_static": (ctypes.c_int, [ctypes.POINTER(GemmArgs), c_void_p]),

@@ -28,7 +28,8 @@ def hipcc_path() -> str:
     return "hipcc"
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, extra_flags: tuple = ()) -> str:
+    """`extra_flags`, e.g. ("-DW4A16_TUNING",), are added to every compile (the planner's tuning overrides)."""
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
     objs = []
     procs = []
@@ -36,7 +37,7 @@ def build(verbose: bool = False) -> str:
     for s in srcs:
         o = s[:-4] + ".o"
         objs.append(o)
-        cmd = [hipcc_path()] + [f for f in HIPCC_FLAGS if f != "-shared"] + ["-c", s, "-o", o]
+        cmd = [hipcc_path()] + [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags) + ["-c", s, "-o", o]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -56,4 +57,4 @@ def build(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, extra_flags=tuple(a for a in sys.argv[1:] if a.startswith("-D"))))

@@ -7,10 +7,16 @@
 
 namespace w4a16 {
 
+// Planner overrides for tuning runs exist only in builds made with -DW4A16_TUNING: W4A16_SPLITS, W4A16_TN and
+// W4A16_KIND (0 general, 1 decode, 2 prefill, 3 64-row, 5 64-row with in-workgroup K split) force the K split count, the
+// decode tile width and the kernel kind; W4A16_DEBUG=1 prints the chosen plan to stderr, =2 every candidate.
+// The shipped library reads no environment variable and prints nothing.
+#ifdef W4A16_TUNING
 static int env_int(const char* name, int dflt) {
   const char* v = getenv(name);
   return (v && *v) ? atoi(v) : dflt;
 }
+#endif
 
 static int validate(const w4a16_gemm_args* a) {
   W4A16_CHECK(a != nullptr, "null args");
@@ -137,12 +143,14 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   }
   pl.total_ksteps = (int)(a->size_k / 32);
   const int cus = num_cus();
-  // Overrides for tuning experiments (unset in production): force the number of K splits, the decode tile width,
-  // or the kernel kind (0 skinny, 1 decode, 2 prefill, 3 64-row); W4A16_DEBUG=1 prints the chosen plan.
+#ifdef W4A16_TUNING
   static const int forced_splits = env_int("W4A16_SPLITS", 0);
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
   static const int debug_plan = env_int("W4A16_DEBUG", 0);
+#else
+  constexpr int forced_splits = 0, forced_tn = 0, forced_kind = -1, debug_plan = 0;
+#endif
 
   // Dense act-order: A's columns are gathered once into a_tmp by permute_cols (as the reference's
   // permute_cols_kernel, csrc/quantization/gptq_marlin/gptq_marlin.cu:68-120), so the GEMM kernels read A with

@@ -19,6 +19,8 @@ namespace w4a16 {
 
 // nibble j of the output word takes source row k0 + DK[j], column n0 + DN[j]
 __device__ __constant__ const int kDK[8] = {0, 8, 0, 8, 1, 9, 1, 9};
+// k-tiles one workgroup of the 4-bit repack kernels walks through (16 KB of output per workgroup)
+constexpr int KT_PER_WG = 16;
 
 // GPTQ source: word (r, n), nibble i = q[8r + i, n].  Without perm a k-tile is two source rows.
 template <bool HAS_PERM>
@@ -30,9 +32,11 @@ __global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __rest
   __shared__ uint32_t tile[HAS_PERM ? 16 : 2][128];
   __shared__ int src_row[16];
   const int t = threadIdx.x;
-  const int kt = blockIdx.y;
   const int ncol0 = blockIdx.x * 128;
   const int ncols = min(128, size_n - ncol0);  // 64 or 128
+  const int kt_end = min((int)(blockIdx.y + 1) * KT_PER_WG, size_k / 16);
+  for (int kt = blockIdx.y * KT_PER_WG; kt < kt_end; ++kt) {
+  __syncthreads();  // the previous k-tile's LDS reads are done
 
   if (HAS_PERM) {
     if (t < 16) src_row[t] = perm[kt * 16 + t];
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __rest
   const int nt = t >> 7;        // n-tile inside the 128-column span
   const int th = (t >> 2) & 31; // "thread" of the Marlin fragment
   const int w = t & 3;
-  if (nt * 64 >= ncols) return;
+  if (nt * 64 < ncols) {
   const int r = 2 * (th & 3);
   const int c = th >> 2;
   const int n0 = nt * 64 + 16 * w + c;
@@ -73,6 +77,8 @@ __global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __rest
     word |= ((src >> (4 * nib)) & 0xFu) << (4 * j);
   }
   out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
+  }
+  }
 }
 
 // AWQ source: word (k, cw), nibble t = q[k, 8*cw + {0,2,4,6,1,3,5,7}[t]]  =>  column 8*cw + j sits
@@ -82,9 +88,11 @@ __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restr
                                                          int size_n) {
   __shared__ uint32_t tile[16][16];  // 16 rows x 16 words (128 columns)
   const int t = threadIdx.x;
-  const int kt = blockIdx.y;
   const int ncol0 = blockIdx.x * 128;
   const int ncols = min(128, size_n - ncol0);
+  const int kt_end = min((int)(blockIdx.y + 1) * KT_PER_WG, size_k / 16);
+  for (int kt = blockIdx.y * KT_PER_WG; kt < kt_end; ++kt) {
+  __syncthreads();  // the previous k-tile's LDS reads are done
   {
     const int row = t >> 4, cw = t & 15;
     if (cw * 8 < ncols) tile[row][cw] = in[(size_t)(kt * 16 + row) * (size_n >> 3) + (ncol0 >> 3) + cw];
@@ -93,7 +101,7 @@ __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restr
   const int nt = t >> 7;
   const int th = (t >> 2) & 31;
   const int w = t & 3;
-  if (nt * 64 >= ncols) return;
+  if (nt * 64 < ncols) {
   const int r = 2 * (th & 3);
   const int c = th >> 2;
   const int n0 = nt * 64 + 16 * w + c;
@@ -107,6 +115,8 @@ __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restr
     word |= ((src >> (4 * nib)) & 0xFu) << (4 * j);
   }
   out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
+  }
+  }
 }
 
 // 8-bit variant (uint8b128): output int32 [K/16, 4N]; per k-tile and n-tile 256 words; word
@@ -154,11 +164,61 @@ __global__ __launch_bounds__(256) void permute_cols_kernel(const uint16_t* __res
     out[(size_t)m * size_k + k] = a[(size_t)m * lda + perm[k]];
 }
 
+// Scale (and bias) permutation of the Marlin layout, 16-bit elements, rows of size_n (a multiple of 64):
+//   grouped:  inside every 64-column chunk, position 8i + j takes the chunk's column i + 8j (an 8 x 8 transpose);
+//   single:   inside every 32-column chunk, position 8i + jj takes column 2i + (jj & 1) + 8 (jj >> 1)
+// (reference marlin_utils.py:278-305).  One thread per output element pair.
+__global__ __launch_bounds__(256) void permute_scales_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
+                                                             int64_t total, int grouped) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int64_t src;
+  if (grouped) {
+    const int p = (int)(idx & 63);
+    src = (idx & ~63LL) + (p >> 3) + 8 * (p & 7);
+  } else {
+    const int p = (int)(idx & 31), i = p >> 3, jj = p & 7;
+    src = (idx & ~31LL) + 2 * i + (jj & 1) + 8 * (jj >> 1);
+  }
+  out[idx] = in[src];
+}
+
+// Zero points -> Marlin packing: output word 8ch + i of a group row (chunk ch of 64 columns), nibble t, holds the
+// zero point of column 64ch + i + 8 * {0,2,4,6,1,3,5,7}[t] (reference marlin_utils.py:326-370).
+// FORMAT 0: packed int32 [G, N/8], nibble j of word c = column 8c + j (compressed-tensors, transposed by the caller);
+// FORMAT 1: AWQ packing, column 8c + j sits in nibble {0,4,1,5,2,6,3,7}[j]; FORMAT 2: unpacked int32 [G, N].
+template <int FORMAT>
+__global__ __launch_bounds__(256) void marlin_zero_points_kernel(const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                                 int64_t total_words, int size_n) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // output word
+  if (idx >= total_words) return;
+  const int words_per_row = size_n >> 3;
+  const int64_t g = idx / words_per_row;
+  const int wi = (int)(idx % words_per_row), ch = wi >> 3, i = wi & 7;
+  uint32_t word = 0;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int m = ((t & 3) << 1) | (t >> 2);  // {0,2,4,6,1,3,5,7}[t]
+    const int col = 64 * ch + i + 8 * m;
+    uint32_t z;
+    if (FORMAT == 2) {
+      z = in[g * size_n + col] & 0xFu;
+    } else {
+      const uint32_t src = in[g * words_per_row + (col >> 3)];
+      const int j = col & 7;
+      const int nib = FORMAT == 1 ? (((j & 1) << 2) | (j >> 1)) : j;
+      z = (src >> (4 * nib)) & 0xFu;
+    }
+    word |= z << (4 * t);
+  }
+  out[idx] = word;
+}
+
 static int check_repack(int64_t size_k, int64_t size_n, int num_bits) {
   W4A16_CHECK(size_k % 16 == 0, "size_k = %lld is not divisible by tile_k_size = 16", (long long)size_k);
   W4A16_CHECK(size_n % 64 == 0, "size_n = %lld is not divisible by tile_n_size = 64", (long long)size_n);
   W4A16_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = %d", num_bits);
-  W4A16_CHECK(size_k / 16 <= 65535, "size_k = %lld too large", (long long)size_k);
+  W4A16_CHECK(size_k / 16 / KT_PER_WG <= 65535, "size_k = %lld too large", (long long)size_k);
   W4A16_CHECK(size_k / 16 * 4 * size_n < (1LL << 31) * 256, "problem too large");
   return 0;
 }
@@ -182,7 +242,7 @@ extern "C" int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
     W4A16_HIP(hipGetLastError());
     return 0;
   }
-  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
+  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)ceil_div(size_k / 16, KT_PER_WG));
   if (perm)
     gptq_repack_kernel<true><<<grid, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n);
   else
@@ -202,7 +262,7 @@ extern "C" int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out
     W4A16_HIP(hipGetLastError());
     return 0;
   }
-  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)(size_k / 16));
+  dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)ceil_div(size_k / 16, KT_PER_WG));
   awq_repack_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k, (int)size_n);
   W4A16_HIP(hipGetLastError());
   return 0;
@@ -220,6 +280,36 @@ extern "C" int w4a16_permute_cols(const void* a, const int32_t* perm, void* out,
     permute_cols_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
         (const uint16_t*)a + m0 * lda, perm, (uint16_t*)out + m0 * size_k, rows, (int)size_k, lda);
   }
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_marlin_permute_scales(const void* s, void* out, int64_t num_rows, int64_t size_n, int grouped,
+                                           void* stream) {
+  W4A16_CHECK(s && out, "null pointer");
+  W4A16_CHECK(size_n % 64 == 0, "size_n = %lld is not divisible by 64", (long long)size_n);
+  const int64_t total = num_rows * size_n;
+  if (total == 0) return 0;
+  W4A16_CHECK(total < (1LL << 31) * 256, "problem too large");
+  permute_scales_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)s, (uint16_t*)out, total, grouped);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_marlin_zero_points(const uint32_t* zp, uint32_t* out, int64_t num_groups, int64_t size_n,
+                                        int format, void* stream) {
+  W4A16_CHECK(zp && out, "null pointer");
+  W4A16_CHECK(size_n % 64 == 0, "size_n = %lld is not divisible by 64", (long long)size_n);
+  W4A16_CHECK(format >= 0 && format <= 2, "unknown zero-point source format %d", format);
+  const int64_t total = num_groups * (size_n / 8);
+  if (total == 0) return 0;
+  W4A16_CHECK(total < (1LL << 31) * 256 && size_n < (1LL << 31), "problem too large");
+  const unsigned blocks = (unsigned)ceil_div(total, 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (format == 0) marlin_zero_points_kernel<0><<<blocks, 256, 0, st>>>(zp, out, total, (int)size_n);
+  if (format == 1) marlin_zero_points_kernel<1><<<blocks, 256, 0, st>>>(zp, out, total, (int)size_n);
+  if (format == 2) marlin_zero_points_kernel<2><<<blocks, 256, 0, st>>>(zp, out, total, (int)size_n);
   W4A16_HIP(hipGetLastError());
   return 0;
 }

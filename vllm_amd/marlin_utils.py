@@ -2,11 +2,10 @@
 vllm/model_executor/layers/quantization/utils/marlin_utils.py (names, arguments and results),
 restricted to what the 4-bit GPTQ / AWQ path needs.  All tensor work runs on the tensor's device.
 """
-import os
-
 import torch
 
 from . import _custom_ops as ops
+from . import _lib
 from .quant_utils import pack_cols, unpack_cols
 from .scalar_type import ScalarType, scalar_types
 
@@ -145,23 +144,51 @@ def get_scale_perms() -> tuple[list[int], list[int]]:
     return scale_perm, scale_perm_single
 
 
-def marlin_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int) -> torch.Tensor:
-    scale_perm, scale_perm_single = get_scale_perms()
-    perm = scale_perm if (group_size < size_k and group_size != -1) else scale_perm_single
+def _device_permute(s: torch.Tensor, grouped: bool) -> torch.Tensor:
+    """One launch of the library's permutation kernel over rows of s.shape[-1] elements."""
+    src = s.contiguous()
+    out = torch.empty_like(src)
+    if src.numel():
+        with torch.cuda.device(src.device):
+            _lib.check(_lib.load().w4a16_marlin_permute_scales(
+                src.data_ptr(), out.data_ptr(), src.numel() // src.shape[-1], src.shape[-1], int(grouped),
+                torch.cuda.current_stream(src.device).cuda_stream))
+    return out
+
+
+def _torch_permute(s: torch.Tensor, perm: list[int], shape) -> torch.Tensor:
     idx = torch.tensor(perm, device=s.device)
-    return s.reshape((-1, len(perm)))[:, idx].reshape((-1, size_n)).contiguous()
+    return s.reshape((-1, len(perm)))[:, idx].reshape(shape).contiguous()
+
+
+def marlin_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int) -> torch.Tensor:
+    """[G, size_n] scales -> Marlin order (reference marlin_utils.py:288-298).  16-bit tensors on the GPU go through
+    one kernel launch; anything else (byte-sized fp4 scales, host tensors) through torch indexing."""
+    grouped = group_size < size_k and group_size != -1
+    if s.is_cuda and s.element_size() == 2 and size_n % 64 == 0:
+        return _device_permute(s.reshape(-1, size_n), grouped)
+    scale_perm, scale_perm_single = get_scale_perms()
+    return _torch_permute(s, scale_perm if grouped else scale_perm_single, (-1, size_n))
 
 
 def marlin_permute_bias(s: torch.Tensor) -> torch.Tensor:
-    _, scale_perm_single = get_scale_perms()
-    idx = torch.tensor(scale_perm_single, device=s.device)
-    return s.reshape((-1, len(scale_perm_single)))[:, idx].reshape(s.shape).contiguous()
+    if s.is_cuda and s.element_size() == 2 and s.shape[-1] % 64 == 0:
+        return _device_permute(s, False)
+    return _torch_permute(s, get_scale_perms()[1], s.shape)
 
 
 def marlin_moe_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int) -> torch.Tensor:
-    out = torch.empty_like(s)
-    for e in range(s.shape[0]):
-        out[e] = marlin_permute_scales(s[e], size_k, size_n, group_size)
+    """All experts in one launch: the permutation works on rows, whichever expert they belong to."""
+    return marlin_permute_scales(s.reshape(-1, size_n), size_k, size_n, group_size).reshape(s.shape)
+
+
+def _device_zero_points(zp: torch.Tensor, num_groups: int, size_n: int, fmt: int) -> torch.Tensor:
+    src = zp.contiguous()
+    out = torch.empty((num_groups, size_n // 8), dtype=torch.int32, device=src.device)
+    if out.numel():
+        with torch.cuda.device(src.device):
+            _lib.check(_lib.load().w4a16_marlin_zero_points(src.data_ptr(), out.data_ptr(), num_groups, size_n, fmt,
+                                                            torch.cuda.current_stream(src.device).cuda_stream))
     return out
 
 
@@ -169,6 +196,8 @@ def marlin_zero_points(zp: torch.Tensor, size_k: int, size_n: int, num_bits: int
     """Unpacked zero points [size_k(=groups), size_n] -> Marlin-packed int32 [groups, size_n/8]
     (marlin_utils.py:326-346)."""
     assert num_bits == 4, "only 4-bit zero points are implemented"
+    if zp.is_cuda and size_n % 64 == 0:
+        return _device_zero_points(zp.reshape(size_k, size_n).to(torch.int32), size_k, size_n, 2)
     scale_perm, _ = get_scale_perms()
     zp = zp.reshape((-1, len(scale_perm)))[:, torch.tensor(scale_perm, device=zp.device)]
     inter = torch.tensor(_INTERLEAVE_4BIT, device=zp.device)
@@ -176,9 +205,20 @@ def marlin_zero_points(zp: torch.Tensor, size_k: int, size_n: int, num_bits: int
     return pack_cols(zp, num_bits, size_k, size_n)
 
 
+def marlin_zero_points_from_packed(zp_packed: torch.Tensor, num_groups: int, size_n: int, num_bits: int) -> torch.Tensor:
+    """Column-packed zero points int32 [groups, size_n/8] (nibble j of word c = column 8c + j) -> Marlin packing.
+    Same result as marlin_zero_points(unpack_cols(zp_packed, ...), ...) without the unpacked intermediate."""
+    assert num_bits == 4, "only 4-bit zero points are implemented"
+    if zp_packed.is_cuda and size_n % 64 == 0:
+        return _device_zero_points(zp_packed, num_groups, size_n, 0)
+    return marlin_zero_points(unpack_cols(zp_packed, num_bits, num_groups, size_n), num_groups, size_n, num_bits)
+
+
 def awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int) -> torch.Tensor:
     """AWQ-packed zero points -> Marlin-packed (marlin_utils.py:349-370)."""
     assert num_bits == 4, "only 4-bit zero points are implemented"
+    if q_zp_packed.is_cuda and size_n % 64 == 0:
+        return _device_zero_points(q_zp_packed, size_k, size_n, 1)
     q_zp = unpack_cols(q_zp_packed, num_bits, size_k, size_n)
     undo = torch.argsort(torch.tensor(_INTERLEAVE_4BIT, device=q_zp.device))
     q_zp = q_zp.reshape((-1, len(_INTERLEAVE_4BIT)))[:, undo].reshape((-1, size_n)).contiguous()
@@ -186,18 +226,25 @@ def awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: in
 
 
 def moe_awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int):
-    out = torch.empty_like(q_zp_packed)
-    for e in range(q_zp_packed.shape[0]):
-        out[e] = awq_to_marlin_zero_points(q_zp_packed[e], size_k, size_n, num_bits)
-    return out
+    """All experts in one launch ([E, groups, size_n/8] is [E * groups, size_n/8] to the kernel)."""
+    e = q_zp_packed.shape[0]
+    return awq_to_marlin_zero_points(q_zp_packed.reshape(e * size_k, -1), e * size_k, size_n, num_bits).reshape(
+        q_zp_packed.shape)
 
 
 def should_use_atomic_add_reduce(m: int, n: int, k: int, device: torch.device, dtype: torch.dtype) -> bool:
-    """marlin_utils.py:412-432.  The flag is forwarded for interface parity; the gfx950 kernels
-    always reduce split-K partials in a fixed order in fp32."""
-    if n >= 2048 or k < 2048 or device.type != "cuda":
-        return False
-    return os.environ.get("VLLM_MARLIN_USE_ATOMIC_ADD", "0") == "1"
+    """Kept for callers that import it (reference marlin_utils.py:412-432).  The gfx950 kernels sum split-K partials in
+    fp32 in a fixed order and have no atomic-add reduction to switch on, so the answer is always False."""
+    return False
+
+
+def _marlin_linear(x: torch.Tensor, weight, scales, zeros, g_idx, sort_indices, workspace, wtype: ScalarType,
+                   size_n: int, size_k: int, is_k_full: bool, bias, use_fp32_reduce: bool) -> torch.Tensor:
+    """[..., size_k] activations through one gptq_marlin_gemm call; leading dimensions are kept."""
+    x2d = x.reshape(-1, x.shape[-1])
+    y = ops.gptq_marlin_gemm(x2d, None, weight, bias, scales, None, zeros, g_idx, sort_indices, workspace, wtype,
+                             x2d.shape[0], size_n, size_k, is_k_full, False, use_fp32_reduce, False)
+    return y.reshape(*x.shape[:-1], size_n)
 
 
 def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
@@ -205,16 +252,9 @@ def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_s
                              workspace: torch.Tensor, wtype: ScalarType, output_size_per_partition: int,
                              input_size_per_partition: int, is_k_full: bool, bias: torch.Tensor | None = None,
                              use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
-    reshaped_x = input.reshape(-1, input.shape[-1])
-    out_shape = input.shape[:-1] + (output_size_per_partition,)
-    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
-                                                  reshaped_x.size(1), input.device, input.dtype)
-    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, weight_zp, g_idx,
-                                  g_idx_sort_indices, workspace, wtype, size_m=reshaped_x.shape[0],
-                                  size_n=output_size_per_partition, size_k=input_size_per_partition,
-                                  is_k_full=is_k_full, use_atomic_add=use_atomic_add,
-                                  use_fp32_reduce=use_fp32_reduce, is_zp_float=False)
-    return output.reshape(out_shape)
+    """Argument list of the reference's function of this name (marlin_utils.py:435-480)."""
+    return _marlin_linear(input, weight, weight_scale, weight_zp, g_idx, g_idx_sort_indices, workspace, wtype,
+                          output_size_per_partition, input_size_per_partition, is_k_full, bias, use_fp32_reduce)
 
 
 def apply_awq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
@@ -222,16 +262,9 @@ def apply_awq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_sc
                             workspace: torch.Tensor, quant_type: ScalarType, output_size_per_partition: int,
                             input_size_per_partition: int, bias: torch.Tensor | None = None,
                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
-    reshaped_x = input.reshape(-1, input.shape[-1])
-    out_shape = input.shape[:-1] + (output_size_per_partition,)
-    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
-                                                  reshaped_x.size(1), input.device, input.dtype)
-    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, weight_zp, g_idx,
-                                  g_idx_sort_indices, workspace, quant_type, size_m=reshaped_x.shape[0],
-                                  size_n=output_size_per_partition, size_k=input_size_per_partition,
-                                  use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,
-                                  is_zp_float=False)
-    return output.reshape(out_shape)
+    """Argument list of the reference's function of this name (marlin_utils.py:483-530); AWQ has no act-order."""
+    return _marlin_linear(input, weight, weight_scale, weight_zp, g_idx, g_idx_sort_indices, workspace, quant_type,
+                          output_size_per_partition, input_size_per_partition, True, bias, use_fp32_reduce)
 
 
 def apply_rtn_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
@@ -239,12 +272,5 @@ def apply_rtn_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_sc
                             input_size_per_partition: int, bias: torch.Tensor | None = None,
                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
     """Round-to-nearest checkpoints: symmetric weights, no zero points, no act-order (marlin_utils.py:533-577)."""
-    reshaped_x = input.reshape(-1, input.shape[-1])
-    out_shape = input.shape[:-1] + (output_size_per_partition,)
-    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), output_size_per_partition,
-                                                  reshaped_x.size(1), input.device, input.dtype)
-    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, None, None, None, workspace,
-                                  quant_type, size_m=reshaped_x.shape[0], size_n=output_size_per_partition,
-                                  size_k=input_size_per_partition, use_atomic_add=use_atomic_add,
-                                  use_fp32_reduce=use_fp32_reduce, is_zp_float=False)
-    return output.reshape(out_shape)
+    return _marlin_linear(input, weight, weight_scale, None, None, None, workspace, quant_type,
+                          output_size_per_partition, input_size_per_partition, True, bias, use_fp32_reduce)

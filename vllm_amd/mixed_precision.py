@@ -8,17 +8,14 @@ Differences: `can_implement` accepts a ROCm gfx950 device instead of requiring C
 are uint4b8, uint8b128 and uint4 + zero points.
 """
 from abc import ABC, abstractmethod
-from collections.abc import Callable
 from dataclasses import dataclass
 
 import torch
 
 from . import _custom_ops as ops
 from .marlin_utils import (MARLIN_SUPPORTED_GROUP_SIZES, apply_gptq_marlin_linear, check_marlin_supports_shape,
-                           marlin_is_k_full, marlin_make_empty_g_idx, marlin_make_workspace_new,
-                           marlin_permute_bias, marlin_permute_scales, marlin_sort_g_idx, marlin_zero_points,
-                           query_marlin_supported_quant_types)
-from .quant_utils import unpack_cols
+                           marlin_is_k_full, marlin_make_workspace_new, marlin_permute_bias, marlin_permute_scales,
+                           marlin_sort_g_idx, marlin_zero_points_from_packed, query_marlin_supported_quant_types)
 from .scalar_type import ScalarType
 
 
@@ -89,18 +86,49 @@ class MPLinearKernel(ABC):
     def apply_weights(self, layer: torch.nn.Module, x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
         raise NotImplementedError
 
-    def _transform_param(self, layer: torch.nn.Module, name: str | None, fn: Callable) -> None:
-        if name is not None and getattr(layer, name, None) is not None:
-            new_param = fn(getattr(layer, name))
-            replace_parameter(layer, name, torch.nn.Parameter(new_param.data, requires_grad=False))
-
     def _get_weight_params(self, layer: torch.nn.Module):
         return (getattr(layer, self.w_q_name), getattr(layer, self.w_s_name),
                 getattr(layer, self.w_zp_name or "", None), getattr(layer, self.w_gidx_name or "", None))
 
 
+@dataclass
+class MarlinLayerTensors:
+    """What the GEMM takes for one layer, all on the weights' device."""
+    qweight: torch.Tensor        # int32 [K/16, N * bits / 2], Marlin layout
+    scales: torch.Tensor         # [G, N], Marlin order
+    zeros: torch.Tensor          # int32 [G, N/8] Marlin packing, or empty
+    g_idx: torch.Tensor          # int32 [K] sorted group of each Marlin row, or empty
+    sort_indices: torch.Tensor   # int32 [K] column gather for the activations, or empty
+    workspace: torch.Tensor
+    is_k_full: bool
+
+
+def prepare_marlin_layer(qweight: torch.Tensor, scales: torch.Tensor, weight_type: ScalarType, size_k: int, size_n: int,
+                         group_size: int, zeros_packed: torch.Tensor | None = None, g_idx: torch.Tensor | None = None,
+                         row_parallel: bool = False) -> MarlinLayerTensors:
+    """Checkpoint tensors of one layer -> GEMM operands, entirely on the device, in four launches at most:
+    the act-order sort (torch), the weight repack, the scale permutation and the zero-point conversion (one kernel of
+    the library each).  qweight: int32 [K / pack, N] packed along K; scales: [G, N]; zeros_packed: int32 [G, N/8]
+    packed along N in natural nibble order; g_idx: int32 [K] group of each input row (act-order) or None."""
+    dev = qweight.device
+    empty = torch.empty(0, dtype=torch.int32, device=dev)
+    sorted_g_idx, sort_indices = (empty, empty) if g_idx is None else marlin_sort_g_idx(g_idx)
+    bits = weight_type.size_bits
+    groups = 1 if group_size == -1 else size_k // group_size
+    return MarlinLayerTensors(
+        qweight=ops.gptq_marlin_repack(qweight.contiguous(), sort_indices, size_k, size_n, bits),
+        scales=marlin_permute_scales(scales.contiguous(), size_k, size_n, group_size),
+        zeros=empty if zeros_packed is None else marlin_zero_points_from_packed(zeros_packed.contiguous(), groups,
+                                                                               size_n, bits),
+        g_idx=sorted_g_idx, sort_indices=sort_indices, workspace=marlin_make_workspace_new(dev),
+        is_k_full=marlin_is_k_full(g_idx is not None, row_parallel))
+
+
 class MarlinLinearKernel(MPLinearKernel):
-    """Repack at load, W4A16 GEMM at apply — both on the gfx950 HIP library."""
+    """Repack at load, W4A16 GEMM at apply, both on the gfx950 HIP library.  Same contract as the reference's class
+    of this name (mixed_precision/marlin.py:28-166): afterwards the layer holds the Marlin-layout weight, scales, zero
+    points and sorted g_idx under the configured parameter names ("w_zp" / "g_idx" when none was given), plus
+    `g_idx_sort_indices`, and a bias, if any, in Marlin order."""
 
     @classmethod
     def get_min_capability(cls) -> int:
@@ -120,63 +148,31 @@ class MarlinLinearKernel(MPLinearKernel):
         return check_marlin_supports_shape(c.partition_weight_shape[1], c.partition_weight_shape[0],
                                            c.full_weight_shape[0], c.group_size)
 
-    # `weight_packed` is brought to {input_dim = 0, output_dim = 1, packed_dim = 0},
-    # `weight_scale` to {input_dim = 0, output_dim = 1}
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
-        device = getattr(layer, self.w_q_name).device
         c = self.config
         size_k, size_n = c.partition_weight_shape
-
-        row_parallel = c.partition_weight_shape[0] != c.full_weight_shape[0]
-        self.is_k_full = marlin_is_k_full(c.has_g_idx, row_parallel)
-        self.workspace = marlin_make_workspace_new(device)
-
-        if self.w_gidx_name is None:
-            self.w_gidx_name = "g_idx"
-        if self.w_zp_name is None:
-            self.w_zp_name = "w_zp"
-
-        if c.has_g_idx:
-            g_idx, g_idx_sort_indices = marlin_sort_g_idx(getattr(layer, self.w_gidx_name))
-            self._transform_param(layer, self.w_gidx_name, lambda _: g_idx)
-            layer.g_idx_sort_indices = g_idx_sort_indices
-        else:
-            setattr(layer, self.w_gidx_name, marlin_make_empty_g_idx(device))
-            layer.g_idx_sort_indices = marlin_make_empty_g_idx(device)
-
-        def transform_w_q(x):
-            w = _to_layout(x, input_dim=0, output_dim=1, packed_dim=0)
-            x.data = ops.gptq_marlin_repack(w.contiguous(), perm=layer.g_idx_sort_indices, size_k=size_k,
-                                            size_n=size_n, num_bits=c.weight_type.size_bits)
-            return x
-
-        def transform_w_s(x):
-            s = _to_layout(x, input_dim=0, output_dim=1)
-            x.data = marlin_permute_scales(s.contiguous(), size_k=size_k, size_n=size_n, group_size=c.group_size)
-            return x
-
-        if c.zero_points:
-            grouped_k = size_k // c.group_size if c.group_size != -1 else 1
-            self._transform_param(
-                layer, self.w_zp_name,
-                lambda x: marlin_zero_points(unpack_cols(x.t(), c.weight_type.size_bits, grouped_k, size_n),
-                                             size_k=grouped_k, size_n=size_n, num_bits=c.weight_type.size_bits))
-        else:
-            setattr(layer, self.w_zp_name, marlin_make_empty_g_idx(device))
-        self._transform_param(layer, self.w_q_name, transform_w_q)
-        self._transform_param(layer, self.w_s_name, transform_w_s)
-
-        if hasattr(layer, "bias") and layer.bias is not None:
-            layer.bias.data = marlin_permute_bias(layer.bias)
+        self.w_gidx_name = self.w_gidx_name or "g_idx"
+        self.w_zp_name = self.w_zp_name or "w_zp"
+        # checkpoint layouts: weight -> [K / pack, N] packed along K, scales -> [G, N], zero points -> [G, N / pack]
+        t = prepare_marlin_layer(
+            _to_layout(getattr(layer, self.w_q_name), input_dim=0, output_dim=1, packed_dim=0),
+            _to_layout(getattr(layer, self.w_s_name), input_dim=0, output_dim=1),
+            c.weight_type, size_k, size_n, c.group_size,
+            zeros_packed=getattr(layer, self.w_zp_name).data.t() if c.zero_points else None,
+            g_idx=getattr(layer, self.w_gidx_name).data if c.has_g_idx else None,
+            row_parallel=size_k != c.full_weight_shape[0])
+        for name, tensor in ((self.w_q_name, t.qweight), (self.w_s_name, t.scales), (self.w_zp_name, t.zeros),
+                             (self.w_gidx_name, t.g_idx), ("g_idx_sort_indices", t.sort_indices)):
+            replace_parameter(layer, name, tensor)
+        self.workspace, self.is_k_full = t.workspace, t.is_k_full
+        if getattr(layer, "bias", None) is not None:
+            layer.bias.data = marlin_permute_bias(layer.bias.data)
 
     def apply_weights(self, layer: torch.nn.Module, x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
-        c = self.config
+        size_k, size_n = self.config.partition_weight_shape
         w_q, w_s, w_zp, w_gidx = self._get_weight_params(layer)
-        return apply_gptq_marlin_linear(
-            input=x, weight=w_q, weight_scale=w_s, weight_zp=w_zp, g_idx=w_gidx,
-            g_idx_sort_indices=layer.g_idx_sort_indices, workspace=self.workspace, wtype=c.weight_type,
-            input_size_per_partition=c.partition_weight_shape[0],
-            output_size_per_partition=c.partition_weight_shape[1], is_k_full=self.is_k_full, bias=bias)
+        return apply_gptq_marlin_linear(x, w_q, w_s, w_zp, w_gidx, layer.g_idx_sort_indices, self.workspace,
+                                        self.config.weight_type, size_n, size_k, self.is_k_full, bias)
 
 
 _POSSIBLE_KERNELS: list[type[MPLinearKernel]] = [MarlinLinearKernel]
