@@ -126,6 +126,13 @@ typedef struct w4a16_gemm_args {
   const void* global_scale;   /* NVFP4 only: [E,] one element of the activation type, as the reference's
                                  nvfp4_marlin_process_global_scale leaves it (marlin_utils_fp4.py:82-93:
                                  x 2^7 for fp16, x 2^119 for bf16); NULL otherwise            */
+  /* ---- fused MoE epilogues (no counterpart in the reference's operator, which runs them as separate launches:
+     fused_marlin_moe.py:47-183, csrc/activation_kernels.cu:85, csrc/moe/moe_align_sum_kernels.cu:375) ---- */
+  void* zero_fill;            /* optional side job of the launch: zero_fill_bytes bytes (a multiple of 16, 16-byte
+                                 aligned) at this address are set to zero; must not overlap any operand of the call */
+  int64_t zero_fill_bytes;
+  int32_t sum_top_k;          /* W4A16_F_SUM_TOPK: result row i is added into c[i / sum_top_k]                     */
+  int32_t reserved2;
 } w4a16_gemm_args;
 
 enum {
@@ -134,9 +141,17 @@ enum {
   W4A16_F_USE_FP32_REDUCE = 4,  /* accepted; partial sums are always fp32                 */
   W4A16_F_MUL_TOPK_WEIGHTS = 8, /* MoE: scale each output row by its routing weight       */
   W4A16_F_MOE = 16,
-  W4A16_F_ZP_FLOAT = 32         /* b_zeros holds fp16 zero points [num_groups, size_n], Marlin-permuted like the
+  W4A16_F_ZP_FLOAT = 32,        /* b_zeros holds fp16 zero points [num_groups, size_n], Marlin-permuted like the
                                    scales (HQQ; reference is_zp_float, gptq_marlin.cu:866-880): w = q*s - zp*s.
                                    fp16, uint4, group size 64, dense op only */
+  W4A16_F_SILU_AND_MUL = 64,    /* MoE only: the weights hold gate | up column halves (size_n = 2 * d, d % 64 == 0);
+                                   c is [size_m * top_k, d] and receives silu(gate) * up, rounded exactly as
+                                   silu_and_mul does on the rounded GEMM result (each of gate, up, silu, product
+                                   rounded once to the activation type) */
+  W4A16_F_SUM_TOPK = 128        /* MoE only: c is [size_m / sum_top_k, size_n], zero on entry (zero_fill of an earlier
+                                   launch on the same stream can do that); every result row i, rounded to the
+                                   activation type, is added to c[i / sum_top_k] with packed 16-bit atomic adds.
+                                   sum_top_k <= 2 (a sum of two rounded terms does not depend on their order) */
 };
 
 /* Bytes of fp32 scratch (c_tmp) a call with these operands may use (0 = none).
@@ -166,6 +181,16 @@ int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int32_t n
                                int32_t block_size, int32_t* sorted_token_ids, int64_t sorted_len,
                                int32_t* expert_ids, int64_t expert_ids_len,
                                int32_t* num_tokens_post_pad, void* stream);
+
+/* Replaces torch.ops._moe_C.batched_moe_align_block_size
+ * (csrc/moe/moe_align_sum_kernels.cu:18-80, 348-373, schema csrc/moe/torch_bindings.cpp:27-34): alignment for
+ * activations already batched per expert.  batch_num_tokens int32 [num_batches <= 1024];
+ * sorted_ids int32 [num_batches * round_up(max_tokens_per_batch, block_size)] (pad value num_batches *
+ * max_tokens_per_batch); block_ids int32 [that / block_size] (-1 past the last block); num_tokens_post_pad int32 [1]. */
+int w4a16_batched_moe_align_block_size(int64_t max_tokens_per_batch, int32_t block_size,
+                                       const int32_t* batch_num_tokens, int32_t num_batches, int32_t* sorted_ids,
+                                       int64_t sorted_len, int32_t* block_ids, int64_t block_ids_len,
+                                       int32_t* num_tokens_post_pad, void* stream);
 
 /* Replaces torch.ops._moe_C.moe_sum (csrc/moe/moe_align_sum_kernels.cu:375-416, schema
  * csrc/moe/torch_bindings.cpp:13): out[t, :] = sum_k in[t, k, :], 16-bit elements, fp32 sum. */

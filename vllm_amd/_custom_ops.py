@@ -5,7 +5,7 @@ PyTorch-ROCm), the operators the reference reaches through `vllm/_custom_ops.py`
 
   _C::gptq_marlin_repack, _C::awq_marlin_repack, _C::gptq_marlin_gemm, _C::permute_cols,
   _C::silu_and_mul, _moe_C::moe_wna16_marlin_gemm, _moe_C::moe_align_block_size, _moe_C::moe_sum,
-  _moe_C::topk_softmax
+  _moe_C::topk_softmax, _moe_C::batched_moe_align_block_size
 
 with the reference's schemas (csrc/torch_bindings.cpp:118, 312-336; csrc/moe/torch_bindings.cpp:13-23, 63-75),
 plus fake (meta) implementations for tracing (reference vllm/_custom_ops.py:553-576, 1179-1218,
@@ -49,6 +49,9 @@ _MOE_SCHEMAS = {
     "moe_wna16_marlin_gemm": _MOE_GEMM_SCHEMA,
     "moe_align_block_size": "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, "
                             "Tensor! sorted_token_ids, Tensor! experts_ids, Tensor! num_tokens_post_pad) -> ()",
+    "batched_moe_align_block_size": "batched_moe_align_block_size(int max_tokens_per_batch, int block_size, "
+                                    "Tensor expert_num_tokens, Tensor! sorted_token_ids, Tensor! experts_ids, "
+                                    "Tensor! num_tokens_post_pad) -> ()",
     "moe_sum": "moe_sum(Tensor input, Tensor! output) -> ()",
     "topk_softmax": "topk_softmax(Tensor! topk_weights, Tensor! topk_indices, Tensor! token_expert_indices, "
                     "Tensor gating_output, bool renormalize) -> ()",
@@ -297,6 +300,29 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
                                 expert_ids, num_tokens_past_padded, topk_weights, moe_block_size, top_k,
                                 mul_topk_weights, is_ep, b_q_type_id, size_m, size_n, size_k, is_full_k,
                                 use_atomic_add, use_fp32_reduce, is_zp_float):
+    return _moe_gemm(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none,
+                     perm_or_none, workspace, sorted_token_ids, expert_ids, num_tokens_past_padded, topk_weights,
+                     moe_block_size, top_k, mul_topk_weights, b_q_type_id, size_m, size_n, size_k, is_full_k,
+                     use_atomic_add, use_fp32_reduce, is_zp_float)
+
+
+def _moe_marlin_gemm_fused_impl(a, c, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none,
+                                g_idx_or_none, perm_or_none, workspace, sorted_token_ids, expert_ids,
+                                num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights,
+                                b_q_type_id, size_m, size_n, size_k, is_full_k, silu_and_mul, sum_top_k, zero_fill):
+    _moe_gemm(a, c, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none, perm_or_none,
+              workspace, sorted_token_ids, expert_ids, num_tokens_past_padded, topk_weights, moe_block_size, top_k,
+              mul_topk_weights, b_q_type_id, size_m, size_n, size_k, is_full_k, False, True, False,
+              silu_and_mul=silu_and_mul, sum_top_k=sum_top_k, zero_fill=zero_fill)
+
+
+def _moe_gemm(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none,
+              perm_or_none, workspace, sorted_token_ids, expert_ids, num_tokens_past_padded, topk_weights,
+              moe_block_size, top_k, mul_topk_weights, b_q_type_id, size_m, size_n, size_k, is_full_k,
+              use_atomic_add, use_fp32_reduce, is_zp_float, silu_and_mul=False, sum_top_k=0, zero_fill=None):
+    """One launch of the MoE GEMM.  silu_and_mul: c is [size_m * top_k, size_n / 2] = silu(gate) * up;
+    sum_top_k > 0: c is [size_m * top_k / sum_top_k, size_n], already zero, and receives the sum of each token's rows;
+    zero_fill: a tensor the launch clears on the side (the output of a later sum_top_k launch)."""
     _check(a.is_cuda and a.is_contiguous() and a.dim() == 2, "A is not a contiguous 2-D GPU tensor")
     _check(a.size(0) == size_m, f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
     _check(a.size(1) == size_k, f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
@@ -355,16 +381,32 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
            "expert_ids is too short for sorted_token_ids")
     _check(topk_weights.is_cuda and topk_weights.dtype == torch.float32 and topk_weights.is_contiguous(),
            "topk_weights must be a contiguous fp32 GPU tensor")
+    c_shape = (size_m * top_k // max(sum_top_k, 1), size_n // 2 if silu_and_mul else size_n)
+    if silu_and_mul:
+        _check(size_n % 128 == 0, f"fused SiLU-and-mul: size_n = {size_n} must be 2 * d with d a multiple of 64")
+    if sum_top_k:
+        _check(sum_top_k in (1, 2) and (size_m * top_k) % sum_top_k == 0, f"unsupported sum_top_k = {sum_top_k}")
     if c_or_none is not None:
         c = c_or_none
         _check(c.is_cuda and c.is_contiguous() and c.dtype == a.dtype, "c is not a contiguous GPU tensor")
-        _check(c.size(0) == size_m * top_k and c.size(1) == size_n, "Shape mismatch: c")
+        _check(tuple(c.shape) == c_shape, "Shape mismatch: c")
     else:
-        c = torch.empty((size_m * top_k, size_n), dtype=a.dtype, device=a.device)
+        _check(not sum_top_k, "the fused top-k sum accumulates into a caller-provided, zeroed c")
+        c = torch.empty(c_shape, dtype=a.dtype, device=a.device)
+    if zero_fill is not None:
+        _check(zero_fill.is_cuda and zero_fill.is_contiguous() and zero_fill.data_ptr() % 16 == 0 and
+               (zero_fill.numel() * zero_fill.element_size()) % 16 == 0,
+               "zero_fill must be a contiguous, 16-byte aligned GPU tensor of a multiple of 16 bytes")
     if size_m == 0:
+        if zero_fill is not None:
+            zero_fill.zero_()
         return c
 
     flags = _lib.F_MOE | (_lib.F_USE_FP32_REDUCE if use_fp32_reduce else 0)
+    if silu_and_mul:
+        flags |= _lib.F_SILU_AND_MUL
+    if sum_top_k:
+        flags |= _lib.F_SUM_TOPK
     if is_full_k:
         flags |= _lib.F_IS_K_FULL
     if use_atomic_add:
@@ -383,6 +425,10 @@ def _moe_wna16_marlin_gemm_impl(a, c_or_none, b_q_weight, b_bias_or_none, b_scal
     args.top_k = top_k
     args.num_experts = num_experts
     args.global_scale = None if gscale is None else gscale.data_ptr()
+    args.sum_top_k = sum_top_k
+    if zero_fill is not None:
+        args.zero_fill = zero_fill.data_ptr()
+        args.zero_fill_bytes = zero_fill.numel() * zero_fill.element_size()
     _run_gemm(args, a.device)
     return c
 
@@ -396,6 +442,19 @@ def _moe_align_block_size_impl(topk_ids, num_experts, block_size, sorted_token_i
         _lib.check(_lib.load().w4a16_moe_align_block_size(
             _ptr(ids), ids.numel(), num_experts, block_size, _ptr(sorted_token_ids), sorted_token_ids.numel(),
             _ptr(experts_ids), experts_ids.numel(), _ptr(num_tokens_post_pad), _stream(topk_ids.device)))
+
+
+def _batched_moe_align_block_size_impl(max_tokens_per_batch, block_size, expert_num_tokens, sorted_token_ids,
+                                       experts_ids, num_tokens_post_pad):
+    _check(expert_num_tokens.is_cuda and expert_num_tokens.is_contiguous() and expert_num_tokens.dim() == 1,
+           "expert_num_tokens must be a contiguous 1-D GPU tensor")
+    n = expert_num_tokens if expert_num_tokens.dtype == torch.int32 else expert_num_tokens.to(torch.int32)
+    for t in (sorted_token_ids, experts_ids, num_tokens_post_pad):
+        _check(t.is_cuda and t.is_contiguous() and t.dtype == torch.int32, "outputs must be contiguous int32 GPU tensors")
+    with torch.cuda.device(n.device):
+        _lib.check(_lib.load().w4a16_batched_moe_align_block_size(
+            max_tokens_per_batch, block_size, _ptr(n), n.numel(), _ptr(sorted_token_ids), sorted_token_ids.numel(),
+            _ptr(experts_ids), experts_ids.numel(), _ptr(num_tokens_post_pad), _stream(n.device)))
 
 
 def _moe_sum_impl(input, output):
@@ -471,11 +530,23 @@ _IMPLS = {
     "_moe_C": {
         "moe_wna16_marlin_gemm": (_moe_wna16_marlin_gemm_impl, _moe_gemm_fake),
         "moe_align_block_size": (_moe_align_block_size_impl, lambda *a: None),
+        "batched_moe_align_block_size": (_batched_moe_align_block_size_impl, lambda *a: None),
         "moe_sum": (_moe_sum_impl, lambda input, output: None),
         "topk_softmax": (_topk_softmax_impl, lambda *a: None),
     },
 }
-_SCHEMAS = {"_C": _C_SCHEMAS, "_moe_C": _MOE_SCHEMAS}
+# Operators of this library's own: the MoE GEMM with a fused epilogue (no counterpart in the reference, which runs
+# silu_and_mul and moe_sum as separate launches).  c, workspace and zero_fill are written.
+_OWN_SCHEMAS = {
+    "moe_marlin_gemm_fused": (
+        "moe_marlin_gemm_fused(Tensor a, Tensor(a!) c, Tensor b_q_weight, Tensor? b_bias_or_none, Tensor b_scales, "
+        "Tensor? global_scale, Tensor? b_zeros_or_none, Tensor? g_idx_or_none, Tensor? perm_or_none, "
+        "Tensor(b!) workspace, Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_past_padded, "
+        "Tensor topk_weights, int moe_block_size, int top_k, bool mul_topk_weights, int b_q_type_id, int size_m, "
+        "int size_n, int size_k, bool is_full_k, bool silu_and_mul, int sum_top_k, Tensor(c!)? zero_fill) -> ()"),
+}
+_IMPLS["w4a16"] = {"moe_marlin_gemm_fused": (_moe_marlin_gemm_fused_impl, lambda *a: None)}
+_SCHEMAS = {"_C": _C_SCHEMAS, "_moe_C": _MOE_SCHEMAS, "w4a16": _OWN_SCHEMAS}
 _libs: list = []          # keep torch.library.Library objects alive
 REGISTERED: list[str] = []  # "ns::op" names this module defined and implemented
 
@@ -557,6 +628,27 @@ def moe_wna16_marlin_gemm(input, output, b_qweight, b_bias, b_scales, global_sca
         sorted_token_ids, expert_ids, num_tokens_past_padded, topk_weights, moe_block_size, top_k,
         mul_topk_weights, is_ep, b_q_type.id, size_m, size_n, size_k, is_k_full, use_atomic_add,
         use_fp32_reduce, is_zp_float)
+
+
+def moe_marlin_gemm_fused(a, c, b_qweight, b_bias, b_scales, global_scale, b_qzeros, g_idx, perm, workspace,
+                          sorted_token_ids, expert_ids, num_tokens_past_padded, topk_weights, moe_block_size: int,
+                          top_k: int, mul_topk_weights: bool, b_q_type: ScalarType, size_m: int, size_n: int,
+                          size_k: int, is_k_full: bool, silu_and_mul: bool = False, sum_top_k: int = 0,
+                          zero_fill: torch.Tensor | None = None) -> None:
+    """The MoE GEMM writing through a fused epilogue into `c`: silu_and_mul -> c [size_m * top_k, size_n / 2];
+    sum_top_k = 2 -> c [size_m * top_k / 2, size_n] (zero on entry) receives each token's two rows added up;
+    zero_fill: a tensor this launch also clears."""
+    torch.ops.w4a16.moe_marlin_gemm_fused(
+        a, c, b_qweight, b_bias, b_scales, global_scale, b_qzeros, g_idx, perm, workspace, sorted_token_ids,
+        expert_ids, num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights, b_q_type.id,
+        size_m, size_n, size_k, is_k_full, silu_and_mul, sum_top_k, zero_fill)
+
+
+def batched_moe_align_block_size(max_tokens_per_batch: int, block_size: int, expert_num_tokens: torch.Tensor,
+                                 sorted_ids: torch.Tensor, expert_ids: torch.Tensor,
+                                 num_tokens_post_pad: torch.Tensor) -> None:
+    torch.ops._moe_C.batched_moe_align_block_size(max_tokens_per_batch, block_size, expert_num_tokens, sorted_ids,
+                                                  expert_ids, num_tokens_post_pad)
 
 
 def permute_cols(a: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:

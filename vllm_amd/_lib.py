@@ -15,6 +15,7 @@ WTYPE_U4B8, WTYPE_U4, WTYPE_U8B128, WTYPE_FE4M3, WTYPE_FE2M1 = 0, 1, 2, 3, 4
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 ABI_VERSION = 3  # W4A16_ABI_VERSION of include/w4a16_gfx950.h this mirror was written against
 F_IS_K_FULL, F_USE_ATOMIC_ADD, F_USE_FP32_REDUCE, F_MUL_TOPK_WEIGHTS, F_MOE, F_ZP_FLOAT = 1, 2, 4, 8, 16, 32
+F_SILU_AND_MUL, F_SUM_TOPK = 64, 128
 
 c_void_p, c_i64, c_i32, c_u32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32
 
@@ -32,6 +33,7 @@ class GemmArgs(ctypes.Structure):
         ("num_tokens_past_padded", c_void_p), ("topk_weights", c_void_p),
         ("n_sorted", c_i64), ("moe_block_size", c_i32), ("top_k", c_i32),
         ("num_experts", c_i32), ("reserved", c_i32), ("global_scale", c_void_p),
+        ("zero_fill", c_void_p), ("zero_fill_bytes", c_i64), ("sum_top_k", c_i32), ("reserved2", c_i32),
     ]
 
 
@@ -48,6 +50,8 @@ EXPORTS = {
     "w4a16_marlin_gemm_static": (ctypes.c_int, [ctypes.POINTER(GemmArgs), c_void_p]),
     "w4a16_moe_align_block_size": (ctypes.c_int, [c_void_p, c_i64, c_i32, c_i32, c_void_p, c_i64, c_void_p,
                                                   c_i64, c_void_p, c_void_p]),
+    "w4a16_batched_moe_align_block_size": (ctypes.c_int, [c_i64, c_i32, c_void_p, c_i32, c_void_p, c_i64, c_void_p,
+                                                          c_i64, c_void_p, c_void_p]),
     "w4a16_moe_sum": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i32, c_i64, c_i32, c_void_p]),
     "w4a16_silu_and_mul": (ctypes.c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i32, c_void_p]),
     "w4a16_topk_softmax": (ctypes.c_int, [c_void_p, c_i32, c_void_p, c_void_p, c_void_p, c_i64, c_i32, c_i32, c_i32,

@@ -81,6 +81,20 @@ static int validate(const w4a16_gemm_args* a) {
                 (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, a->g_idx != nullptr,
                 (long long)a->num_groups);
   }
+  if (a->flags & (W4A16_F_SILU_AND_MUL | W4A16_F_SUM_TOPK))
+    W4A16_CHECK((a->flags & W4A16_F_MOE) != 0, "the fused SiLU-and-mul / top-k sum epilogues exist for the MoE GEMM only");
+  if (a->flags & W4A16_F_SILU_AND_MUL) {
+    W4A16_CHECK(a->size_n % 128 == 0, "fused SiLU-and-mul: size_n = %lld must be 2 * d with d a multiple of 64",
+                (long long)a->size_n);
+    W4A16_CHECK(!(a->flags & W4A16_F_SUM_TOPK), "fused SiLU-and-mul and the top-k sum cannot be combined");
+  }
+  if (a->flags & W4A16_F_SUM_TOPK)
+    W4A16_CHECK(a->sum_top_k == 1 || a->sum_top_k == 2, "fused top-k sum: sum_top_k = %d must be 1 or 2", a->sum_top_k);
+  if (a->zero_fill)
+    W4A16_CHECK((a->flags & W4A16_F_MOE) != 0, "zero_fill is a side job of the MoE GEMM only");
+  if (a->zero_fill)
+    W4A16_CHECK(a->zero_fill_bytes >= 0 && a->zero_fill_bytes % 16 == 0 && ((uintptr_t)a->zero_fill & 15) == 0,
+                "zero_fill must be 16-byte aligned and a multiple of 16 bytes long");
   if (a->flags & W4A16_F_MOE) {
     W4A16_CHECK(a->sorted_token_ids && a->expert_ids && a->num_tokens_past_padded, "null MoE index pointer");
     W4A16_CHECK(a->moe_block_size == 8 || (a->moe_block_size % 16 == 0 && a->moe_block_size >= 16 &&
@@ -296,6 +310,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     for (int ti = 0; ti < n_tn; ++ti) {
       const int tn = ti == 0 ? 128 : 64;
       if (forced_tn && tn != forced_tn && decode_ok) continue;
+      if (tn == 64 && (a->flags & W4A16_F_SILU_AND_MUL)) continue;  // gate and up n-tiles are paired in 128-column tiles
       const int64_t ncol_tiles = ceil_div(a->size_n, tn);
       const int64_t tiles = mtiles * ncol_tiles;
       if (tiles <= 0 || tiles >= (1LL << 31) / 64) continue;

@@ -59,6 +59,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     }
   }
   const int ct = tile % p.ncp, mt = tile / p.ncp;  // column tile, m-tile
+  zero_fill_side_job(p);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
@@ -122,8 +123,8 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
 
   // n-tile this lane reads (TN=128: 2ct+h, TN=64: ct); a missing second n-tile (N/64 odd) aliases n-tile 0
   int nt;
-  if (TN == 128)
-    nt = (2 * ct + h) * 64 < p.N ? 2 * ct + h : 0;
+  if (TN == 128)  // (fused SiLU-and-mul: gate n-tile ct paired with the up n-tile of the same output columns)
+    nt = p.act ? (h ? (p.N >> 7) + ct : ct) : ((2 * ct + h) * 64 < p.N ? 2 * ct + h : 0);
   else
     nt = ct;
   const int64_t b_row = (int64_t)p.N * 2;  // words per k-tile row
@@ -320,10 +321,9 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   const bool single = p.splits == 1;
   float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (16 * TN);
 
-  auto finalize = [&](float* v) {
-    const int crow = s_crow[fr];
-    if (crow < 0 || !fcol_ok) return;
-    const int base = ncol & ~31, cl = ncol & 31;
+  // channel scale, bias and routing weight of CPT finished columns starting at real column `col`
+  auto finish = [&](float* v, int col, int crow) {
+    const int base = col & ~31, cl = col & 31;
     if (CHANNEL) {
 #pragma unroll
       for (int j = 0; j < CPT; ++j) {
@@ -343,10 +343,41 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
 #pragma unroll
       for (int j = 0; j < CPT; ++j) v[j] *= tw;
     }
-    uint16_t* dst = (uint16_t*)p.C + (int64_t)crow * p.N + ncol;
-#pragma unroll
-    for (int j = 0; j < CPT; j += 2)
-      *(uint32_t*)(dst + j) = (DT == DT_F16) ? pack_f16(v[j], v[j + 1]) : pack_bf16(v[j], v[j + 1]);
+  };
+  // fused SiLU-and-mul (TN = 128 only, host-checked): the threads of the gate half also take the up half's columns
+  const bool act_lane = TN == 128 && p.act && fc < 64;
+  auto finalize = [&](float* v, float* u) {
+    const int crow = s_crow[fr];
+    if (crow < 0) return;
+    if constexpr (TN == 128) {
+      if (p.act) {
+        if (!act_lane) return;
+        const int oc = ct * 64 + fc;
+        finish(v, oc, crow);
+        finish(u, (p.N >> 1) + oc, crow);
+        store_row4_silu_mul<DT>(p, crow, oc, f32x4{v[0], v[1], v[2], v[3]}, f32x4{u[0], u[1], u[2], u[3]});
+        return;
+      }
+    }
+    if (!fcol_ok) return;
+    finish(v, ncol, crow);
+    if constexpr (CPT == 4) {
+      store_row4<DT>(p, crow, ncol, f32x4{v[0], v[1], v[2], v[3]});
+    } else {
+      const uint32_t o = pack2<DT>(v[0], v[1]);
+      if (p.sum_div > 0) {
+        uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * p.N + ncol;
+        if constexpr (DT == DT_F16) {
+          typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+          __builtin_amdgcn_global_atomic_fadd_v2f16((h2*)dst, __builtin_bit_cast(h2, o));
+        } else {
+          typedef short s2 __attribute__((ext_vector_type(2)));
+          __builtin_amdgcn_global_atomic_fadd_v2bf16((s2*)dst, __builtin_bit_cast(s2, o));
+        }
+      } else {
+        *(uint32_t*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+      }
+    }
   };
 
   __syncthreads();  // A bounce slabs no longer read
@@ -361,9 +392,9 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
         for (int r = 0; r < 4; ++r) mine[(4 * g + r) * RS + HS * h + 16 * w + 8 * hf + c] = acc[w][hf][r];
   }
   __syncthreads();
-  float v[CPT];
+  float v[CPT], u[CPT];
 #pragma unroll
-  for (int j = 0; j < CPT; ++j) v[j] = 0.0f;
+  for (int j = 0; j < CPT; ++j) v[j] = u[j] = 0.0f;
 #pragma unroll
   for (int ww = 0; ww < DNW; ++ww) {
     const float* src = red + ww * (16 * RS) + fr * RS + fpos;
@@ -371,7 +402,15 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     for (int j = 0; j < CPT; ++j) v[j] += src[j];
   }
   if (single) {
-    finalize(v);
+    if (act_lane) {
+#pragma unroll
+      for (int ww = 0; ww < DNW; ++ww) {
+        const float* src = red + ww * (16 * RS) + fr * RS + fpos + 72;
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) u[j] += src[j];
+      }
+    }
+    finalize(v, u);
     return;
   }
   if (s_crow[fr] >= 0) {
@@ -385,26 +424,30 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   __syncthreads();
   if (!s_last) return;
   if (s_crow[fr] >= 0) {
-    const float* parts = p.ctmp + (int64_t)tile * p.splits * (16 * TN) + fr * TN + fc;
+    auto sum_parts = [&](float* out, int col) {
+      const float* parts = p.ctmp + (int64_t)tile * p.splits * (16 * TN) + fr * TN + col;
 #pragma unroll
-    for (int j = 0; j < CPT; ++j) v[j] = 0.0f;
-    // four splits' loads are in flight together (a loop of dependent round trips would cost ~0.3 us per split)
-    for (int s0 = 0; s0 < p.splits; s0 += 4) {
-      float a[4][CPT];
+      for (int j = 0; j < CPT; ++j) out[j] = 0.0f;
+      // four splits' loads are in flight together (a loop of dependent round trips would cost ~0.3 us per split)
+      for (int s0 = 0; s0 < p.splits; s0 += 4) {
+        float a[4][CPT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int s = min(s0 + i, p.splits - 1);
+        for (int i = 0; i < 4; ++i) {
+          const int s = min(s0 + i, p.splits - 1);
 #pragma unroll
-        for (int j = 0; j < CPT; j += 2) load_coherent2(parts + (int64_t)s * (16 * TN) + j, a[i][j], a[i][j + 1]);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (s0 + i < p.splits) {
-#pragma unroll
-          for (int j = 0; j < CPT; ++j) v[j] += a[i][j];
+          for (int j = 0; j < CPT; j += 2) load_coherent2(parts + (int64_t)s * (16 * TN) + j, a[i][j], a[i][j + 1]);
         }
-    }
-    finalize(v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (s0 + i < p.splits) {
+#pragma unroll
+            for (int j = 0; j < CPT; ++j) out[j] += a[i][j];
+          }
+      }
+    };
+    sum_parts(v, fc);
+    if (act_lane) sum_parts(u, fc + 64);
+    finalize(v, u);
   }
 }
 

@@ -39,7 +39,67 @@ struct KParams {
   int moe, moe_bs, top_k, mul_topk;
   int n_sorted;  // usable length of sorted_ids
   int64_t b_estride, s_estride, z_estride, k_estride, n_estride;  // per-expert strides (elements)
+  // fused epilogues
+  int act;        // 1: column halves are gate | up; C is [rows, N / 2] = silu(gate) * up
+  int sum_div;    // > 0: result row i is added atomically into C row i / sum_div
+  uint32_t* zero_ptr;  // side job: zero_n16 16-byte pieces to clear, spread over the grid
+  int64_t zero_n16;
 };
+
+// Side job of a launch: the grid clears `zero_n16` 16-byte pieces at `zero_ptr` (the output of a later launch that
+// accumulates with atomic adds).  Every workgroup of the grid calls this first, before any early exit.
+__device__ __forceinline__ void zero_fill_side_job(const KParams& p) {
+  if (p.zero_n16 <= 0) return;
+  const int64_t per = (p.zero_n16 + gridDim.x - 1) / gridDim.x;
+  const int64_t b = (int64_t)blockIdx.x * per, e = b + per < p.zero_n16 ? b + per : p.zero_n16;
+  for (int64_t i = b + threadIdx.x; i < e; i += blockDim.x) ((u32x4*)p.zero_ptr)[i] = u32x4{0, 0, 0, 0};
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return DT == DT_F16 ? pack_f16(lo, hi) : pack_bf16(lo, hi);
+}
+template <int DT>
+__device__ __forceinline__ float lo_f32(uint32_t x) { return DT == DT_F16 ? f16_lo_f32(x) : bf16_lo_f32(x); }
+template <int DT>
+__device__ __forceinline__ float hi_f32(uint32_t x) { return DT == DT_F16 ? f16_hi_f32(x) : bf16_hi_f32(x); }
+
+// Four finished fp32 results of C row `crow`, columns ncol .. ncol + 3: rounded to the 16-bit type, then stored, or
+// (sum_div > 0) added into row crow / sum_div with packed 16-bit atomic adds.
+template <int DT>
+__device__ __forceinline__ void store_row4(const KParams& p, int crow, int ncol, f32x4 v) {
+  const uint32_t o0 = pack2<DT>(v[0], v[1]), o1 = pack2<DT>(v[2], v[3]);
+  if (p.sum_div > 0) {
+    uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * p.N + ncol;
+    if constexpr (DT == DT_F16) {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      __builtin_amdgcn_global_atomic_fadd_v2f16((h2*)dst, __builtin_bit_cast(h2, o0));
+      __builtin_amdgcn_global_atomic_fadd_v2f16((h2*)(dst + 2), __builtin_bit_cast(h2, o1));
+    } else {
+      typedef short s2 __attribute__((ext_vector_type(2)));
+      __builtin_amdgcn_global_atomic_fadd_v2bf16((s2*)dst, __builtin_bit_cast(s2, o0));
+      __builtin_amdgcn_global_atomic_fadd_v2bf16((s2*)(dst + 2), __builtin_bit_cast(s2, o1));
+    }
+  } else {
+    *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = u32x2{o0, o1};
+  }
+}
+
+// silu(gate) * up on finished fp32 results, with the roundings of a GEMM store followed by the reference's
+// act_and_mul_kernel<silu> (csrc/activation_kernels.cu:22-40): gate and up rounded to the 16-bit type, SiLU evaluated
+// in fp32 and rounded, the product rounded.  Stored at C[crow][ocol .. ocol + 3], row stride N / 2.
+template <int DT>
+__device__ __forceinline__ void store_row4_silu_mul(const KParams& p, int crow, int ocol, f32x4 gate, f32x4 up) {
+  float r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t gu = pack2<DT>(gate[j], up[j]);
+    const float gv = lo_f32<DT>(gu), uv = hi_f32<DT>(gu);
+    const float sv = gv / (1.0f + expf(-gv));
+    r[j] = lo_f32<DT>(pack2<DT>(sv, 0.f)) * uv;
+  }
+  *(u32x2*)((uint16_t*)p.C + (int64_t)crow * (p.N >> 1) + ocol) = u32x2{pack2<DT>(r[0], r[1]), pack2<DT>(r[2], r[3])};
+}
 
 // Split-K partials cross XCDs (each XCD has its own L2).  A plain store stays dirty in the writer's L2,
 // and an agent-scope release fence (an L2 write-back) costs ~0.5 us per workgroup, serialised per L2.
@@ -146,6 +206,10 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.z_estride = a->num_groups * (a->size_n / 8);
   p.k_estride = a->size_k;
   p.n_estride = a->size_n;
+  p.act = moe && (a->flags & W4A16_F_SILU_AND_MUL);
+  p.sum_div = (moe && (a->flags & W4A16_F_SUM_TOPK)) ? a->sum_top_k : 0;
+  p.zero_ptr = (uint32_t*)a->zero_fill;
+  p.zero_n16 = a->zero_fill ? a->zero_fill_bytes / 16 : 0;
   return p;
 }
 

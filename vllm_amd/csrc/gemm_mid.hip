@@ -61,6 +61,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
   const int row0 = mt * MD_BM;
+  zero_fill_side_job(p);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
@@ -97,7 +98,8 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   }
 
   // ---- weights of this wavefront
-  const int nt = (wave_on && (2 * cp + h) * 64 < p.N) ? 2 * cp + h : 0;
+  // (fused SiLU-and-mul: gate n-tile cp paired with the up n-tile of the same output columns, N/128 + cp)
+  const int nt = !wave_on ? 0 : (MOE && p.act) ? (h ? (p.N >> 7) + cp : cp) : ((2 * cp + h) * 64 < p.N ? 2 * cp + h : 0);
   // 4-bit: 32 u32x4 per n-tile and k-tile, one per Marlin thread; 8-bit: 64, two per thread (words 2w + half)
   const int64_t b_row = (BITS == 4) ? (p.N >> 1) : p.N;
   const u32x4* bp = (const u32x4*)Bq + nt * (8 * BITS) + (4 * c + g) * (BITS / 4);
@@ -315,27 +317,39 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const int fpos = fc4 + (fc4 >= 64 ? 8 : 0);
   const int ncol = cp * 128 + fc4;
   const bool fcol_ok = wave_on && ncol < p.N;
-  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool act = MOE && p.act;
+  const bool act_lane = act && fc4 < 64;
+  // cs / bs: channel (and global) scale and bias of the thread's four columns; cu / bu: of the up half's columns
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f}, cu[4] = {1.f, 1.f, 1.f, 1.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
   if constexpr (FP4 == 1) {
     // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
     const uint16_t gv = *gscale;
     const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) cs[j] = gs;
+    for (int j = 0; j < 4; ++j) cs[j] = cu[j] = gs;
   }
-  if (fcol_ok) {
-    const int base = ncol & ~31, cl = ncol & 31;
+  auto col_consts = [&](int col, float* sc_out, float* b_out) {
+    const int base = col & ~31, cl = col & 31;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (CHANNEL) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        cs[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
+        sc_out[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
       if (bias) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
-        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+        b_out[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
       }
     }
+  };
+  const int ocol = cp * 64 + fc4;  // fused SiLU-and-mul: output column of a gate-half thread
+  if (act) {
+    if (act_lane && wave_on) {
+      col_consts(ocol, cs, bs);
+      col_consts((p.N >> 1) + ocol, cu, bu);
+    }
+  } else if (fcol_ok) {
+    col_consts(ncol, cs, bs);
   }
 #pragma unroll
   for (int mb = 0; mb < MD_MB; ++mb) {
@@ -358,7 +372,26 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
           *(f32x4*)(p.ctmp + (((int64_t)tile * p.splits + split) * MD_BM + mb * 16 + r16) * 512 + wv * 128 + fc4) = v;
         continue;
       }
-      if (fcol_ok && crow >= 0) {
+      if (crow < 0) continue;
+      if (act) {
+        if (act_lane && wave_on) {
+          f32x4 u = *(const f32x4*)(slab + r16 * RED_RS + fpos + 72);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[j] = v[j] * cs[j] + bs[j];
+            u[j] = u[j] * cu[j] + bu[j];
+          }
+          if (p.mul_topk) {
+            const float tw = p.topk_w[crow];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              v[j] *= tw;
+              u[j] *= tw;
+            }
+          }
+          store_row4_silu_mul<DT>(p, crow, ocol, v, u);
+        }
+      } else if (fcol_ok) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
         if (MOE && p.mul_topk) {
@@ -366,12 +399,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] *= tw;
         }
-        u32x2 o;
-        if constexpr (DT == DT_F16)
-          o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
-        else
-          o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-        *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+        store_row4<DT>(p, crow, ncol, v);
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -400,29 +428,35 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
     if (bias) bias += e * p.n_estride;
   }
   const int fc4 = (t & 127) * 4;
-  const int ncol = nt4 * 512 + fc4;
-  if (ncol >= p.N) return;
-  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool act = MOE && p.act;
+  // fused SiLU-and-mul: the 128 columns of wavefront block fc4 / 128 are 64 gate columns followed by the 64 up columns
+  // of the same outputs; only the gate half's threads finish rows
+  const int cp = nt4 * 4 + (fc4 >> 7);
+  const int ncol = act ? cp * 64 + (fc4 & 127) : nt4 * 512 + fc4;
+  if (act ? ((fc4 & 127) >= 64 || cp * 128 >= p.N) : ncol >= p.N) return;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f}, cu[4] = {1.f, 1.f, 1.f, 1.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
   if (gscale) {
     const uint16_t gv = *gscale;
     const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) cs[j] = gs;
+    for (int j = 0; j < 4; ++j) cs[j] = cu[j] = gs;
   }
-  {
-    const int base = ncol & ~31, cl = ncol & 31;
+  auto col_consts = [&](int col, float* sc_out, float* b_out) {
+    const int base = col & ~31, cl = col & 31;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (CHANNEL) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        cs[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
+        sc_out[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (p.fp8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
       if (bias) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
-        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+        b_out[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
       }
     }
-  }
+  };
+  col_consts(ncol, cs, bs);
+  if (act) col_consts((p.N >> 1) + ncol, cu, bu);
   const float* parts = p.ctmp + (int64_t)tile * p.splits * (MD_BM * 512) + fc4;
 #pragma unroll 2
   for (int i = 0; i < 8; ++i) {
@@ -435,21 +469,27 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
       crow = row0 + r;
     }
     if (crow < 0) continue;
-    f32x4 v = {0, 0, 0, 0};
+    f32x4 v = {0, 0, 0, 0}, u = {0, 0, 0, 0};
     for (int sidx = 0; sidx < p.splits; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512);
+    if (act)
+      for (int sidx = 0; sidx < p.splits; ++sidx) u += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512 + 64);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+    for (int j = 0; j < 4; ++j) {
+      v[j] = v[j] * cs[j] + bs[j];
+      u[j] = u[j] * cu[j] + bu[j];
+    }
     if (MOE && p.mul_topk) {
       const float tw = p.topk_w[crow];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] *= tw;
+      for (int j = 0; j < 4; ++j) {
+        v[j] *= tw;
+        u[j] *= tw;
+      }
     }
-    u32x2 o;
-    if constexpr (DT == DT_F16)
-      o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+    if (act)
+      store_row4_silu_mul<DT>(p, crow, ncol, v, u);
     else
-      o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-    *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+      store_row4<DT>(p, crow, ncol, v);
   }
 }
 

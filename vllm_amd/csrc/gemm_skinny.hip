@@ -84,6 +84,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     }
   }
   const int cp = tile % p.ncp, mt = tile / p.ncp;
+  zero_fill_side_job(p);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
@@ -150,7 +151,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const int nks = w_e - w_b;
 
   // lanes of an n-tile past the end of N (odd number of n-tiles) read n-tile 0; their columns are never stored
-  const int nt = (2 * cp + h) * 64 < p.N ? 2 * cp + h : 0;
+  // (fused SiLU-and-mul: the tile pairs gate n-tile cp with the up n-tile of the same output columns, N/128 + cp)
+  const int nt = p.act ? (h ? (p.N >> 7) + cp : cp) : ((2 * cp + h) * 64 < p.N ? 2 * cp + h : 0);
   // 4-bit: 32 u32x4 per n-tile and k-tile, one per Marlin thread; 8-bit: 64, two per thread (words 2w + half)
   const int64_t b_row = (BITS == 4) ? (p.N >> 1) : p.N;  // u32x4 per k-tile row
   const u32x4* bp = (const u32x4*)Bq + nt * (8 * BITS) + (4 * c + g) * (BITS / 4);
@@ -456,11 +458,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const bool single = p.splits == 1;
   float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (BM * 128);
 
-  auto finalize = [&](int r, f32x4 v) {
-    const int crow = s_crow[r];
-    if (crow < 0 || !fcol_ok) return;
+  // channel scale, global scale, bias and routing weight of four finished columns starting at real column `col`
+  auto finish = [&](f32x4 v, int col, int crow) {
     if (GM == GM_CHANNEL) {
-      const int base = ncol & ~31, cl = ncol & 31;
+      const int base = col & ~31, cl = col & 31;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
@@ -475,7 +476,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       for (int j = 0; j < 4; ++j) v[j] *= gs;
     }
     if (bias) {
-      const int base = ncol & ~31, cl = ncol & 31;
+      const int base = col & ~31, cl = col & 31;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint16_t bv = bias[base + single_perm_pos(cl + j)];
@@ -487,12 +488,20 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] *= tw;
     }
-    u32x2 o;
-    if constexpr (DT == DT_F16)
-      o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
-    else
-      o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-    *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+    return v;
+  };
+  // v: the thread's four columns; u (fused SiLU-and-mul, threads of the gate half only): the up half's same columns
+  const bool act_lane = p.act && fc4 < 64;
+  auto finalize = [&](int r, f32x4 v, f32x4 u) {
+    const int crow = s_crow[r];
+    if (crow < 0) return;
+    if (p.act) {
+      if (!act_lane) return;
+      const int oc = cp * 64 + fc4;
+      store_row4_silu_mul<DT>(p, crow, oc, finish(v, oc, crow), finish(u, (p.N >> 1) + oc, crow));
+    } else if (fcol_ok) {
+      store_row4<DT>(p, crow, ncol, finish(v, ncol, crow));
+    }
   };
 
 #pragma unroll
@@ -513,10 +522,16 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 #pragma unroll
     for (int ww = 1; ww < NW; ++ww) v += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos);
     const int r = mb * 16 + fr;
-    if (single)
-      finalize(r, v);
-    else if (s_crow[r] >= 0)
+    if (single) {
+      f32x4 u = {0, 0, 0, 0};
+      if (act_lane) {
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) u += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos + 72);
+      }
+      finalize(r, v, u);
+    } else if (s_crow[r] >= 0) {
       store_coherent(my_part + r * 128 + fc4, v);
+    }
   }
   if (single) return;
 
@@ -528,21 +543,27 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   __syncthreads();
   if (!s_last) return;
   const float* parts = p.ctmp + (int64_t)tile * p.splits * (BM * 128);
-#pragma unroll 1
-  for (int r = fr; r < BM; r += 16) {
-    if (s_crow[r] < 0) continue;
+  auto sum_parts = [&](int r, int col4) {
     f32x4 v = {0, 0, 0, 0};
     // four splits' loads are in flight together; summed in split order
     for (int s0 = 0; s0 < p.splits; s0 += 4) {
       f32x4 a[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        a[i] = load_coherent(parts + (int64_t)min(s0 + i, p.splits - 1) * (BM * 128) + r * 128 + fc4);
+        a[i] = load_coherent(parts + (int64_t)min(s0 + i, p.splits - 1) * (BM * 128) + r * 128 + col4);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (s0 + i < p.splits) v += a[i];
     }
-    finalize(r, v);
+    return v;
+  };
+#pragma unroll 1
+  for (int r = fr; r < BM; r += 16) {
+    if (s_crow[r] < 0) continue;
+    const f32x4 v = sum_parts(r, fc4);
+    f32x4 u = {0, 0, 0, 0};
+    if (act_lane) u = sum_parts(r, fc4 + 64);
+    finalize(r, v, u);
   }
 }
 

@@ -237,6 +237,51 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
 
 using namespace w4a16;
 
+// Alignment for activations already batched per expert ([B, max_tokens, K], batch_num_tokens[b] valid rows in batch
+// b), the contract of the reference's batched_moe_align_block_size (csrc/moe/moe_align_sum_kernels.cu:18-80, 348-373):
+// batch b's rows b * max_tokens + j, j < n_b, padded to a multiple of block_size with the value B * max_tokens, runs
+// packed in batch order; one batch id per block, -1 past the last; the padded total.  One workgroup: an inclusive scan
+// of the padded counts in LDS, then every output slot is written exactly once (its batch found by bisection).
+__global__ __launch_bounds__(ALIGN_THREADS) void batched_moe_align_kernel(
+    int num_batches, int max_tokens, int block_size, const int32_t* __restrict__ batch_num_tokens,
+    int32_t* __restrict__ sorted_ids, int sorted_len, int32_t* __restrict__ block_ids, int32_t* __restrict__ num_post_pad) {
+  __shared__ int incl[ALIGN_MAX_EXPERTS];  // inclusive scan of padded counts
+  __shared__ int cnt[ALIGN_MAX_EXPERTS];
+  const int t = threadIdx.x;
+  const int n = t < num_batches ? min(max(batch_num_tokens[t], 0), max_tokens) : 0;
+  cnt[t] = n;
+  incl[t] = (n + block_size - 1) / block_size * block_size;
+  __syncthreads();
+  for (int d = 1; d < ALIGN_THREADS; d <<= 1) {
+    const int add = t >= d ? incl[t - d] : 0;
+    __syncthreads();
+    incl[t] += add;
+    __syncthreads();
+  }
+  const int total = incl[ALIGN_THREADS - 1];
+  if (t == 0) *num_post_pad = total;
+  const int sentinel = num_batches * max_tokens;
+  auto batch_of = [&](int pos) {  // first b with incl[b] > pos (pos < total)
+    int lo = 0, hi = num_batches - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (incl[mid] > pos) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+  };
+  for (int i = t; i < sorted_len; i += ALIGN_THREADS) {
+    int v = sentinel;
+    if (i < total) {
+      const int b = batch_of(i);
+      const int start = b == 0 ? 0 : incl[b - 1];
+      if (i - start < cnt[b]) v = b * max_tokens + (i - start);
+    }
+    sorted_ids[i] = v;
+  }
+  for (int i = t; i < sorted_len / block_size; i += ALIGN_THREADS)
+    block_ids[i] = i * block_size < total ? batch_of(i * block_size) : -1;
+}
+
 extern "C" int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int32_t num_experts,
                                           int32_t block_size, int32_t* sorted_token_ids, int64_t sorted_len,
                                           int32_t* expert_ids, int64_t expert_ids_len,
@@ -311,6 +356,26 @@ extern "C" int w4a16_topk_softmax(const void* gating_output, int32_t gating_dtyp
                                                     token_expert_indices, (int)num_tokens, num_experts, topk, renormalize);
   else
     return fail(W4A16_EINVAL, "gating_output must be fp16, bf16 or fp32");
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int w4a16_batched_moe_align_block_size(int64_t max_tokens_per_batch, int32_t block_size,
+                                                  const int32_t* batch_num_tokens, int32_t num_batches,
+                                                  int32_t* sorted_ids, int64_t sorted_len, int32_t* block_ids,
+                                                  int64_t block_ids_len, int32_t* num_tokens_post_pad, void* stream) {
+  W4A16_CHECK(batch_num_tokens && sorted_ids && block_ids && num_tokens_post_pad, "null pointer");
+  W4A16_CHECK(block_size > 0 && max_tokens_per_batch >= 0, "bad block_size / max_tokens_per_batch");
+  W4A16_CHECK(num_batches >= 1 && num_batches <= ALIGN_MAX_EXPERTS, "num_batches = %d must be in [1, %d]", num_batches,
+              ALIGN_MAX_EXPERTS);
+  const int64_t want = ceil_div(max_tokens_per_batch, block_size) * block_size * num_batches;
+  W4A16_CHECK(sorted_len == want, "sorted_ids has %lld elements, expected %lld", (long long)sorted_len, (long long)want);
+  W4A16_CHECK(block_ids_len == want / block_size, "batch_ids has %lld elements, expected %lld", (long long)block_ids_len,
+              (long long)(want / block_size));
+  W4A16_CHECK(want < (1LL << 31) && num_batches * max_tokens_per_batch < (1LL << 31), "problem too large");
+  batched_moe_align_kernel<<<1, ALIGN_THREADS, 0, (hipStream_t)stream>>>(num_batches, (int)max_tokens_per_batch, block_size,
+                                                                         batch_num_tokens, sorted_ids, (int)sorted_len,
+                                                                         block_ids, num_tokens_post_pad);
   W4A16_HIP(hipGetLastError());
   return 0;
 }

@@ -1,7 +1,24 @@
-"""Fused MoE on the Marlin-layout W4A16 kernels; host choreography with the reference's signature
-(vllm/model_executor/layers/fused_moe/fused_marlin_moe.py:47-340): block-size pick, token alignment,
-GEMM1 (gate|up) -> SiLU-and-mul -> GEMM2 (down, scaled by routing weights) -> sum over top-k."""
+"""Mixture-of-experts layer over Marlin-layout expert weights on the gfx950 MoE GEMM.
+
+Public functions keep the reference's names and argument lists
+(vllm/model_executor/layers/fused_moe/fused_marlin_moe.py: `fused_marlin_moe` :186-340,
+`batched_fused_marlin_moe` :343-498), so a caller written against the reference works unchanged.
+The launch sequence is this library's own.  Where the reference runs five launches
+
+    align -> GEMM1 -> silu_and_mul -> GEMM2 (x routing weight) -> moe_sum,
+
+the default path here runs three:
+
+    align -> GEMM1 with SiLU-and-mul in its epilogue (and the final output cleared on the side)
+          -> GEMM2 x routing weight, each token's top-k rows added into the output by the epilogue.
+
+The [tokens * topk, 2 * inter] GEMM1 result and the [tokens, topk, hidden] GEMM2 result never reach memory.  Results
+are those of the five-launch sequence (the epilogues round where the separate kernels would have).  The five-launch
+sequence remains for what the fused epilogues do not cover: a caller-supplied activation or sum function, more than
+two experts per token.
+"""
 from collections.abc import Callable
+from dataclasses import dataclass
 
 import torch
 
@@ -10,57 +27,115 @@ from .marlin_utils import marlin_make_workspace_new, marlin_moe_intermediate_siz
 from .moe_align_block_size import batched_moe_align_block_size, moe_align_block_size
 from .scalar_type import ScalarType, scalar_types
 
+_MOE_WEIGHT_TYPES = (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn,
+                     scalar_types.float4_e2m1f)
+_BLOCK_SIZES = (8, 16, 32, 48, 64)  # token slots per expert block the MoE GEMM accepts
+
 
 def default_activation_func(activation: str, output: torch.Tensor, input: torch.Tensor) -> None:
-    if activation == "silu":
-        ops.silu_and_mul(output, input)
-    else:
+    if activation != "silu":
         raise ValueError(f"Unsupported activation: {activation}. Only silu is implemented.")
+    ops.silu_and_mul(output, input)
 
 
-def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk: int,
-                      quant_type: ScalarType, apply_router_weight_on_input: bool, expert_map, block_size_m: int,
-                      sorted_token_ids, expert_ids, num_tokens_post_padded, activation: str = "silu",
-                      activation_func: Callable = default_activation_func, global_scale1=None, global_scale2=None,
-                      g_idx1=None, g_idx2=None, sort_indices1=None, sort_indices2=None, w1_zeros=None, w2_zeros=None,
-                      workspace=None, intermediate_cache13=None, intermediate_cache2=None, output=None,
-                      is_k_full: bool = True) -> torch.Tensor:
-    assert hidden_states.ndim == 2
-    M, K = hidden_states.size()
-    N = marlin_moe_intermediate_size(w1, w2)
-    if workspace is None:
-        workspace = marlin_make_workspace_new(hidden_states.device, 4)
-    if intermediate_cache13 is None:
-        intermediate_cache13 = torch.empty((M * num_topk * max(2 * N, K),), device=hidden_states.device,
-                                           dtype=hidden_states.dtype)
-    if intermediate_cache2 is None:
-        intermediate_cache2 = torch.empty((M * num_topk, N), device=hidden_states.device, dtype=hidden_states.dtype)
-    cache1 = intermediate_cache13[:M * num_topk * 2 * N].view(M * num_topk, 2 * N)
-    cache3 = intermediate_cache13[:M * num_topk * K].view(M * num_topk, K)
-    cache2 = intermediate_cache2.view(-1)[:M * num_topk * N].view(M * num_topk, N)
-    use_atomic_add = hidden_states.dtype == torch.half
+def pick_block_size(tokens: int, topk: int, num_experts: int) -> int:
+    """Smallest block that the average expert's share of the token slots fills to less than 90 %
+    (the reference's rule, fused_marlin_moe.py:279-282), else the largest."""
+    per_expert = tokens * topk / num_experts
+    return next((bs for bs in _BLOCK_SIZES if per_expert < 0.9 * bs), _BLOCK_SIZES[-1])
 
-    cache1 = ops.moe_wna16_marlin_gemm(
-        hidden_states, cache1, w1, bias1, w1_scale, global_scale1, w1_zeros, g_idx1, sort_indices1, workspace,
-        sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
-        top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, is_ep=expert_map is not None,
-        b_q_type=quant_type, size_m=M, size_n=2 * N, size_k=K, is_k_full=is_k_full,
-        use_atomic_add=use_atomic_add, use_fp32_reduce=True, is_zp_float=False)
 
-    activation_func(activation, cache2, cache1.view(-1, 2 * N))
+@dataclass
+class _Experts:
+    """The operands that stay the same across the two GEMMs of one layer call."""
+    quant_type: ScalarType
+    w: tuple            # (w1, w2)
+    scale: tuple
+    bias: tuple
+    global_scale: tuple
+    zeros: tuple
+    g_idx: tuple
+    sort_indices: tuple
+    is_k_full: bool
+    workspace: torch.Tensor
 
-    if output is None:
-        output = cache3
-    if expert_map is not None:
-        output.zero_()
+    def operands(self, i: int):
+        return (self.w[i], self.bias[i], self.scale[i], self.global_scale[i], self.zeros[i], self.g_idx[i],
+                self.sort_indices[i])
 
-    output = ops.moe_wna16_marlin_gemm(
-        cache2, output, w2, bias2, w2_scale, global_scale2, w2_zeros, g_idx2, sort_indices2, workspace,
-        sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
-        top_k=1, mul_topk_weights=not apply_router_weight_on_input, is_ep=expert_map is not None,
-        b_q_type=quant_type, size_m=M * num_topk, size_n=K, size_k=N, is_k_full=is_k_full,
-        use_atomic_add=use_atomic_add, use_fp32_reduce=True, is_zp_float=False)
-    return output
+
+@dataclass
+class _Routing:
+    sorted_token_ids: torch.Tensor
+    expert_ids: torch.Tensor
+    num_tokens_post_padded: torch.Tensor
+    topk_weights: torch.Tensor
+    block_size: int
+    topk: int
+    expert_parallel: bool
+
+
+def _gemm(ex: _Experts, which: int, rt: _Routing, a, c, size_m, size_n, size_k, top_k, mul_weights, **fused):
+    w, bias, scale, gscale, zeros, g_idx, sort_idx = ex.operands(which)
+    common = (a, c, w, bias, scale, gscale, zeros, g_idx, sort_idx, ex.workspace, rt.sorted_token_ids, rt.expert_ids,
+              rt.num_tokens_post_padded, rt.topk_weights, rt.block_size, top_k, mul_weights)
+    if fused:
+        ops.moe_marlin_gemm_fused(*common, ex.quant_type, size_m, size_n, size_k, ex.is_k_full, **fused)
+        return c
+    return ops.moe_wna16_marlin_gemm(*common, rt.expert_parallel, ex.quant_type, size_m, size_n, size_k, ex.is_k_full,
+                                     a.dtype == torch.half, True, False)
+
+
+def _run_experts(x: torch.Tensor, ex: _Experts, rt: _Routing, weight_on_input: bool, activation: str,
+                 activation_func: Callable, moe_sum: Callable | None, out: torch.Tensor | None, inter_buf, gemm_buf,
+                 reduce_topk: bool) -> torch.Tensor:
+    """x [M, K] -> [M, K] (reduce_topk) or [M * topk, K].  `out` receives the result when given."""
+    m, k = x.shape
+    n = marlin_moe_intermediate_size(*ex.w)
+    slots = m * rt.topk
+    dev, dt = x.device, x.dtype
+    act = inter_buf.view(-1)[:slots * n].view(slots, n) if inter_buf is not None else torch.empty((slots, n), device=dev, dtype=dt)
+    fusable = activation == "silu" and activation_func is default_activation_func and moe_sum is None
+    if fusable and (rt.topk <= 2 or not reduce_topk):
+        if out is None:
+            out = torch.empty((m if reduce_topk else slots, k), device=dev, dtype=dt)
+        summing = reduce_topk and rt.topk == 2
+        needs_zero = summing or rt.expert_parallel       # rows of experts on other ranks are never written
+        aliased = out is x                                # inplace: GEMM1 still reads what the side job would clear
+        side_job = out if needs_zero and not aliased and out.is_contiguous() else None
+        _gemm(ex, 0, rt, x, act, m, 2 * n, k, rt.topk, weight_on_input, silu_and_mul=True, sum_top_k=0, zero_fill=side_job)
+        if needs_zero and side_job is None:
+            out.zero_()
+        _gemm(ex, 1, rt, act, out, slots, k, n, 1, not weight_on_input, silu_and_mul=False,
+              sum_top_k=2 if summing else 0, zero_fill=None)
+        return out
+    # general sequence: separate activation and top-k sum
+    big = max(2 * n, k)
+    shared = gemm_buf if gemm_buf is not None else torch.empty((slots * big,), device=dev, dtype=dt)
+    h = _gemm(ex, 0, rt, x, shared.view(-1)[:slots * 2 * n].view(slots, 2 * n), m, 2 * n, k, rt.topk, weight_on_input)
+    activation_func(activation, act, h)
+    y = shared.view(-1)[:slots * k].view(slots, k) if reduce_topk or out is None else out
+    if rt.expert_parallel:
+        y.zero_()
+    y = _gemm(ex, 1, rt, act, y, slots, k, n, 1, not weight_on_input)
+    if not reduce_topk:
+        return y
+    if out is None:
+        out = torch.empty((m, k), device=dev, dtype=dt)
+    y3 = y.view(m, rt.topk, k)
+    if moe_sum is None:
+        ops.moe_sum(y3, out)
+        return out
+    return moe_sum(y3, out)
+
+
+def _check_layer(hidden_2d_k: int, w1, w2, quant_type: ScalarType, dtype) -> None:
+    assert quant_type in _MOE_WEIGHT_TYPES, f"unsupported MoE weight type {quant_type}"
+    assert w1.size(1) * 16 == hidden_2d_k, "Hidden size mismatch w1"
+    assert w2.size(2) // (quant_type.size_bits // 2) == hidden_2d_k, "Hidden size mismatch w2"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert dtype in (torch.float16, torch.bfloat16)
 
 
 def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, gating_output, topk_weights,
@@ -71,53 +146,26 @@ def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, ga
                      sort_indices1=None, sort_indices2=None, w1_zeros=None, w2_zeros=None, workspace=None,
                      intermediate_cache13=None, intermediate_cache2=None, is_k_full: bool = True, output=None,
                      inplace: bool = False) -> torch.Tensor:
-    """Mixture-of-experts layer over Marlin-layout 4-bit expert weights w1 [E, K/16, 2*(2N)] and
-    w2 [E, N/16, 2*K]; returns [M, K]."""
-    if inplace:
-        assert output is None, "Conflicting request"
-    quant_type = ScalarType.from_id(quant_type_id)
-    assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
-                          scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f), \
-        f"unsupported MoE weight type {quant_type}"
-    num_bits = quant_type.size_bits
-    M, K = hidden_states.size()
-    E = w1.size(0)
-    topk = topk_ids.size(1)
-    if gating_output is not None:
-        assert gating_output.size(0) == M, "Number of tokens mismatch"
-    assert w1.size(1) * 16 == K, "Hidden size mismatch w1"
-    assert w2.size(2) // (num_bits // 2) == K, "Hidden size mismatch w2"
-    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
-    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
-    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
-    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    """hidden_states [M, K]; w1 [E, K/16, 2N * bits/2] (gate | up), w2 [E, N/16, K * bits/2] in Marlin layout;
+    topk_weights fp32 [M, topk], topk_ids [M, topk]; returns [M, K]."""
+    assert not (inplace and output is not None), "Conflicting request"
+    assert hidden_states.ndim == 2 and hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert topk_weights.dtype == torch.float32
-
-    for block_size_m in (8, 16, 32, 48, 64):
-        if M * topk / E / block_size_m < 0.9:
-            break
-    if global_num_experts == -1:
-        global_num_experts = E
-    sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
-        topk_ids, block_size_m, global_num_experts, expert_map)
-
-    moe_output = _fused_marlin_moe(
-        hidden_states=hidden_states, w1=w1, w2=w2, bias1=bias1, bias2=bias2, w1_scale=w1_scale, w2_scale=w2_scale,
-        topk_weights=topk_weights, num_topk=topk, quant_type=quant_type,
-        apply_router_weight_on_input=apply_router_weight_on_input, expert_map=expert_map,
-        block_size_m=block_size_m, sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
-        num_tokens_post_padded=num_tokens_post_padded, activation=activation, activation_func=activation_func,
-        global_scale1=global_scale1, global_scale2=global_scale2, g_idx1=g_idx1, g_idx2=g_idx2,
-        sort_indices1=sort_indices1, sort_indices2=sort_indices2, w1_zeros=w1_zeros, w2_zeros=w2_zeros,
-        workspace=workspace, intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2,
-        output=None, is_k_full=is_k_full).view(-1, topk, K)
-
-    if output is None:
-        output = hidden_states if inplace else torch.empty_like(hidden_states)
-    if moe_sum is None:
-        ops.moe_sum(moe_output.contiguous(), output)
-        return output
-    return moe_sum(moe_output, output)
+    m, k = hidden_states.shape
+    assert gating_output is None or gating_output.size(0) == m, "Number of tokens mismatch"
+    quant_type = ScalarType.from_id(quant_type_id)
+    _check_layer(k, w1, w2, quant_type, hidden_states.dtype)
+    num_local = w1.size(0)
+    topk = topk_ids.size(1)
+    bs = pick_block_size(m, topk, num_local)
+    sorted_ids, expert_ids, post_pad = moe_align_block_size(
+        topk_ids, bs, num_local if global_num_experts == -1 else global_num_experts, expert_map)
+    ex = _Experts(quant_type, (w1, w2), (w1_scale, w2_scale), (bias1, bias2), (global_scale1, global_scale2),
+                  (w1_zeros, w2_zeros), (g_idx1, g_idx2), (sort_indices1, sort_indices2), is_k_full,
+                  workspace if workspace is not None else marlin_make_workspace_new(hidden_states.device, 4))
+    rt = _Routing(sorted_ids, expert_ids, post_pad, topk_weights, bs, topk, expert_map is not None)
+    return _run_experts(hidden_states, ex, rt, apply_router_weight_on_input, activation, activation_func, moe_sum,
+                        hidden_states if inplace else output, intermediate_cache2, intermediate_cache13, True)
 
 
 def batched_fused_marlin_moe(hidden_states, expert_num_tokens, w1, w2, bias1, bias2, w1_scale, w2_scale, gating_output,
@@ -127,45 +175,27 @@ def batched_fused_marlin_moe(hidden_states, expert_num_tokens, w1, w2, bias1, bi
                              sort_indices2=None, w1_zeros=None, w2_zeros=None, workspace=None,
                              intermediate_cache13=None, intermediate_cache2=None, is_k_full: bool = True, output=None,
                              inplace: bool = False) -> torch.Tensor:
-    """MoE over activations already batched per expert, hidden_states [E, max_tokens, K] with expert_num_tokens[e]
-    valid rows in batch e (reference fused_marlin_moe.py:343-498): the batch is viewed as [E * max_tokens, K] with
-    top_k = 1 and unit routing weights, and the alignment comes from the row counts.  Returns [E, max_tokens, K];
-    rows past expert_num_tokens[e] are not written."""
+    """Activations already batched per expert: hidden_states [E, max_tokens, K] with expert_num_tokens[e] valid rows in
+    batch e.  The batch is the flat [E * max_tokens, K] problem with one expert per token and unit routing weights;
+    the alignment comes from the row counts.  Returns [E, max_tokens, K]; rows past expert_num_tokens[e] are not written."""
     assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K]. But got {hidden_states.size()}"
-    if inplace:
-        assert output is None, "Conflicting request."
-    quant_type = ScalarType.from_id(quant_type_id)
-    assert quant_type in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
-                          scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f), \
-        f"unsupported MoE weight type {quant_type}"
-    num_bits = quant_type.size_bits
-    B, batch_tokens_max, K = hidden_states.size()
-    M = B * batch_tokens_max
-    E = w1.size(0)
+    assert not (inplace and output is not None), "Conflicting request."
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
-    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
-    assert expert_num_tokens.size(0) == E
-    assert B == E, "Batch must be as big as number of experts as the tokens are sorted into the batch/expert they belong to"
-    assert w1.size(1) * 16 == K, "Hidden size mismatch w1"
-    assert w2.size(2) // (num_bits // 2) == K, "Hidden size mismatch w2"
-    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
-    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
     assert activation is not None
-    topk = 1
-    block_size_m = 64
-    sorted_token_ids, expert_ids, num_tokens_post_padded = batched_moe_align_block_size(
-        max_tokens_per_batch=batch_tokens_max, block_size=block_size_m, expert_num_tokens=expert_num_tokens)
-    if output is None and inplace:
-        output = hidden_states
-    topk_weights = torch.ones((M, topk), device=hidden_states.device, dtype=torch.float32)
-    output = _fused_marlin_moe(
-        hidden_states=hidden_states.view(-1, K), w1=w1, w2=w2, bias1=bias1, bias2=bias2, w1_scale=w1_scale,
-        w2_scale=w2_scale, topk_weights=topk_weights, num_topk=topk, quant_type=quant_type,
-        apply_router_weight_on_input=apply_router_weight_on_input, activation=activation, expert_map=expert_map,
-        block_size_m=block_size_m, sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
-        num_tokens_post_padded=num_tokens_post_padded, global_scale1=global_scale1, global_scale2=global_scale2,
-        g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2, w1_zeros=w1_zeros,
-        w2_zeros=w2_zeros, workspace=workspace, intermediate_cache13=intermediate_cache13,
-        intermediate_cache2=intermediate_cache2, output=output.view(-1, K) if output is not None else output,
-        is_k_full=is_k_full)
-    return output.view(B, batch_tokens_max, K)
+    batches, max_tokens, k = hidden_states.shape
+    quant_type = ScalarType.from_id(quant_type_id)
+    _check_layer(k, w1, w2, quant_type, hidden_states.dtype)
+    assert expert_num_tokens.size(0) == w1.size(0) == batches, \
+        "Batch must be as big as number of experts as the tokens are sorted into the batch/expert they belong to"
+    bs = _BLOCK_SIZES[-1]
+    sorted_ids, expert_ids, post_pad = batched_moe_align_block_size(max_tokens, bs, expert_num_tokens)
+    flat = hidden_states.view(-1, k)
+    ones = torch.ones((flat.size(0), 1), device=flat.device, dtype=torch.float32)
+    ex = _Experts(quant_type, (w1, w2), (w1_scale, w2_scale), (bias1, bias2), (global_scale1, global_scale2),
+                  (w1_zeros, w2_zeros), (g_idx1, g_idx2), (sort_indices1, sort_indices2), is_k_full,
+                  workspace if workspace is not None else marlin_make_workspace_new(flat.device, 4))
+    rt = _Routing(sorted_ids, expert_ids, post_pad, ones, bs, 1, expert_map is not None)
+    dest = flat if inplace else (output.view(-1, k) if output is not None else None)
+    y = _run_experts(flat, ex, rt, apply_router_weight_on_input, activation, default_activation_func, None, dest,
+                     intermediate_cache2, intermediate_cache13, False)
+    return y.view(batches, max_tokens, k)

@@ -33,27 +33,13 @@ def batched_moe_align_block_size(max_tokens_per_batch: int, block_size: int,
     expert_num_tokens[e] valid rows in batch e; same result contract as the reference's function of this name
     (vllm/model_executor/layers/fused_moe/moe_align_block_size.py:88-172): row index e * max_tokens_per_batch + j
     for the valid rows of expert e, each expert padded to a multiple of block_size with the value
-    E * max_tokens_per_batch, experts with no tokens skipped, expert_ids = -1 past the last block.
-    Computed with a handful of torch integer ops on the device (no host synchronisation)."""
+    E * max_tokens_per_batch, experts with no tokens skipped, expert_ids = -1 past the last block."""
     e = expert_num_tokens.size(0)
     dev = expert_num_tokens.device
-    padded = -(-max_tokens_per_batch // block_size) * block_size
-    nb_max = padded // block_size
-    sentinel = e * max_tokens_per_batch
-    n = expert_num_tokens.to(torch.int64)
-    nblk = (n + block_size - 1) // block_size
-    off = torch.cumsum(nblk, 0) - nblk                                    # first block of every expert
-    eb = torch.arange(e, device=dev).view(e, 1, 1)
-    b = torch.arange(nb_max, device=dev).view(1, nb_max, 1)
-    j = torch.arange(block_size, device=dev).view(1, 1, block_size)
-    live = b < nblk.view(e, 1, 1)
-    tok = b * block_size + j
-    val = torch.where(tok < n.view(e, 1, 1), eb * max_tokens_per_batch + tok, sentinel)
-    dest = torch.where(live, (off.view(e, 1, 1) + b) * block_size + j, e * padded)   # dead blocks -> spare slot
-    sorted_ext = torch.full((e * padded + 1,), sentinel, dtype=torch.int32, device=dev)
-    sorted_ext.scatter_(0, dest.reshape(-1), val.reshape(-1).to(torch.int32))
-    ids_ext = torch.full((e * nb_max + 1,), -1, dtype=torch.int32, device=dev)
-    dest_b = torch.where(live[:, :, 0], off.view(e, 1) + b[:, :, 0], e * nb_max)
-    ids_ext.scatter_(0, dest_b.reshape(-1), eb[:, :, 0].expand(e, nb_max).reshape(-1).to(torch.int32))
-    total = (nblk.sum() * block_size).to(torch.int32).view(1)
-    return sorted_ext[:-1], ids_ext[:-1], total
+    padded = e * (-(-max_tokens_per_batch // block_size) * block_size)
+    sorted_ids = torch.empty((padded,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((padded // block_size,), dtype=torch.int32, device=dev)
+    num_tokens_post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+    ops.batched_moe_align_block_size(max_tokens_per_batch, block_size, expert_num_tokens, sorted_ids, expert_ids,
+                                     num_tokens_post_pad)
+    return sorted_ids, expert_ids, num_tokens_post_pad
