@@ -72,6 +72,9 @@ def test_silu_and_mul(dev, dtype, m, d):
     eps = 2.0 ** (-10 if dtype == torch.float16 else -7)
     assert ((got - want).abs() <= eps * want.abs() + 1e-6).all()
     assert torch.allclose(got, mr.silu_and_mul(x.float()), rtol=4 * eps, atol=1e-3)
+    # the reference's own bar (tests/kernels/core/test_activation.py:93-97): exactly the native PyTorch result on the device
+    xd = x.to(dev)
+    assert torch.equal(out, torch.nn.functional.silu(xd[:, :d]) * xd[:, d:])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])

@@ -501,6 +501,12 @@ __device__ __forceinline__ void raw_pair(uint32_t xa, uint32_t xb, u32x4& o0, u3
   }
 }
 
+// SiLU in fp32 exactly as PyTorch's device kernel and the reference's act_and_mul_kernel evaluate it
+// (csrc/activation_kernels.cu:28-32): x / (1 + expf(-x)) with the correctly rounded quotient, so that results equal
+// torch.nn.functional.silu on the same device bit for bit (the reference tests this op for exact equality,
+// tests/kernels/core/test_activation.py:93-97).
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
 // Position of real column `cl` (0..31 inside its 32-column chunk) in a tensor permuted with the
 // reference's "single" permutation (marlin_utils.py:278-286, used for channel-wise scales and bias).
 __device__ __forceinline__ int single_perm_pos(int cl) {

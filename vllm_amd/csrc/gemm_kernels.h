@@ -95,8 +95,7 @@ __device__ __forceinline__ void store_row4_silu_mul(const KParams& p, int crow, 
   for (int j = 0; j < 4; ++j) {
     const uint32_t gu = pack2<DT>(gate[j], up[j]);
     const float gv = lo_f32<DT>(gu), uv = hi_f32<DT>(gu);
-    const float sv = gv / (1.0f + expf(-gv));
-    r[j] = lo_f32<DT>(pack2<DT>(sv, 0.f)) * uv;
+    r[j] = lo_f32<DT>(pack2<DT>(silu_f32(gv), 0.f)) * uv;
   }
   *(u32x2*)((uint16_t*)p.C + (int64_t)crow * (p.N >> 1) + ocol) = u32x2{pack2<DT>(r[0], r[1]), pack2<DT>(r[2], r[3])};
 }

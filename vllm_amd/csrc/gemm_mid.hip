@@ -318,7 +318,6 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const int ncol = cp * 128 + fc4;
   const bool fcol_ok = wave_on && ncol < p.N;
   const bool act = MOE && p.act;
-  const bool act_lane = act && fc4 < 64;
   // cs / bs: channel (and global) scale and bias of the thread's four columns; cu / bu: of the up half's columns
   float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f}, cu[4] = {1.f, 1.f, 1.f, 1.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
   if constexpr (FP4 == 1) {
@@ -342,9 +341,12 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       }
     }
   };
-  const int ocol = cp * 64 + fc4;  // fused SiLU-and-mul: output column of a gate-half thread
+  // fused SiLU-and-mul, unsplit: lane -> row (lane >> 4) + 4 i, gate columns 4 (lane & 15) .. + 3 and the up columns of
+  // the same outputs, so that all 64 lanes take part
+  const int ac4 = (lane & 15) * 4;
+  const int ocol = cp * 64 + ac4;
   if (act) {
-    if (act_lane && wave_on) {
+    if (wave_on) {
       col_consts(ocol, cs, bs);
       col_consts((p.N >> 1) + ocol, cu, bu);
     }
@@ -360,6 +362,32 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) slab[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
     __builtin_amdgcn_wave_barrier();
+    if (act && p.splits == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r16 = (lane >> 4) + 4 * i;
+        const int crow = s_crow[mb * 16 + r16];
+        if (crow < 0 || !wave_on) continue;
+        f32x4 v = *(const f32x4*)(slab + r16 * RED_RS + ac4);
+        f32x4 u = *(const f32x4*)(slab + r16 * RED_RS + ac4 + 72);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] = v[j] * cs[j] + bs[j];
+          u[j] = u[j] * cu[j] + bu[j];
+        }
+        if (p.mul_topk) {
+          const float tw = p.topk_w[crow];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[j] *= tw;
+            u[j] *= tw;
+          }
+        }
+        store_row4_silu_mul<DT>(p, crow, ocol, v, u);
+      }
+      __builtin_amdgcn_wave_barrier();
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int r16 = (lane >> 5) + 2 * i;
@@ -373,25 +401,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
         continue;
       }
       if (crow < 0) continue;
-      if (act) {
-        if (act_lane && wave_on) {
-          f32x4 u = *(const f32x4*)(slab + r16 * RED_RS + fpos + 72);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            v[j] = v[j] * cs[j] + bs[j];
-            u[j] = u[j] * cu[j] + bu[j];
-          }
-          if (p.mul_topk) {
-            const float tw = p.topk_w[crow];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              v[j] *= tw;
-              u[j] *= tw;
-            }
-          }
-          store_row4_silu_mul<DT>(p, crow, ocol, v, u);
-        }
-      } else if (fcol_ok) {
+      if (fcol_ok) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
         if (MOE && p.mul_topk) {

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
       yv[1] = DT == DT_F16 ? f16_hi_f32(y[j]) : bf16_hi_f32(y[j]);
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        const float s = xv[q] / (1.0f + expf(-xv[q]));
+        const float s = silu_f32(xv[q]);
         const uint32_t sr = DT == DT_F16 ? pack_f16(s, 0.f) : pack_bf16(s, 0.f);
         const float st = DT == DT_F16 ? f16_lo_f32(sr) : bf16_lo_f32(sr);
         r[q] = st * yv[q];
