@@ -115,3 +115,45 @@ def test_linear_kernel_w8(dev):
     out = kern.apply_weights(layer, x.to(dev))
     mt = gr.error_metrics(out, gr.gemm_ref(x, w_ref))
     assert mt["max_rel"] <= 2e-2 and mt["mean_rel"] < 0.04, mt
+
+
+@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 4, 8), (33, 2, 8, 16), (123, 3, 4, 32), (333, 2, 4, 64)])
+@pytest.mark.parametrize("dtype,k_full", [(torch.float16, True), (torch.bfloat16, True), (torch.float16, False)])
+def test_moe_gemm_w8_act_order(ops, dev, dtype, k_full, m, topk, e, bs):
+    """uint8b128 experts with act-order (per-expert g_idx and column gather inside the kernel), which the reference
+    instantiates for its MoE op (csrc/moe/marlin_moe_wna16/ops.cu:441); against the per-slot oracle, and one-hot rows
+    bit-exactly."""
+    from oracle import gemm_ref as gr
+    from oracle import moe_ref as mr
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    k, n = 256, 192
+    layers = [make_layer(k, n, 32, dtype, act_order=True, seed=70 + i, w_std=0.1, bits=8) for i in range(e)]
+    st = lambda name: torch.stack([getattr(l, name) for l in layers]).to(dev)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+    tw = torch.rand(m, topk, generator=g)
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e)
+    ws = marlin_make_workspace_new(dev, 4)
+
+    def run(a):
+        return ops.moe_wna16_marlin_gemm(
+            a.to(dev), None, st("marlin_q"), None, st("marlin_s"), None, None, st("g_idx_sorted"), st("sort_indices"), ws,
+            s, x, t, tw.to(dev), moe_block_size=bs, top_k=topk, mul_topk_weights=False, is_ep=False,
+            b_q_type=scalar_types.uint8b128, size_m=m, size_n=n, size_k=k, is_k_full=k_full, use_atomic_add=False,
+            use_fp32_reduce=True, is_zp_float=False)
+    a = torch.randn(m, k, generator=g).to(dtype)
+    out = run(a)
+    w_dense = torch.stack([l.w_ref for l in layers])
+    ref = mr.moe_gemm_ref(a, w_dense, s.cpu(), x.cpu(), t.cpu(), tw, bs, topk, False, m)
+    mt = gr.error_metrics(out, ref)
+    assert mt["max_rel"] <= (2e-2 if dtype == torch.float16 else 4e-2) and mt["mean_rel"] < 0.04, mt
+    ks = torch.randint(0, k, (m,), generator=g)
+    hot = torch.zeros(m, k, dtype=dtype)
+    hot[torch.arange(m), ks] = 1.0
+    out = run(hot).cpu()
+    for i in range(m):
+        for j in range(topk):
+            assert torch.equal(out[i * topk + j], layers[int(ids[i, j])].w_ref[ks[i]])
+    assert int(ws.abs().sum()) == 0

@@ -56,5 +56,80 @@ def build(verbose: bool = False, extra_flags: tuple = ()) -> str:
     return LIB_PATH
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# MFMAs issued through inline assembly (gemm_fat.hip, gemm_mid.hip, gemm_kq.hip) are opaque to the compiler's hazard
+# logic.  On gfx950 an MFMA that reads a register fewer than two wait states after a VALU instruction wrote it sees
+# the old value.  The kernels keep their operand writes far from the MFMAs that read them; this check compiles the
+# files to assembly (device pass only, no GPU needed) and reports every MFMA whose A, B or C operand is written by a
+# VALU instruction (v_accvgpr_write included) with fewer than two wait states in between (every instruction counts
+# one, `s_nop N` counts N + 1).
+ASM_MFMA_SOURCES = ["gemm_fat.hip", "gemm_mid.hip", "gemm_kq.hip"]
+
+
+def _regs(tok: str) -> set:
+    import re
+    m = re.match(r"([va])\[(\d+):(\d+)\]", tok)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.match(r"([va])(\d+)$", tok)
+    return {(m.group(1), int(m.group(2)))} if m else set()
+
+
+def scan_mfma_hazards(asm_path: str):
+    """Returns (number of MFMAs seen, list of (writer, mfma) instruction pairs that are too close)."""
+    total, bad = 0, []
+    hist = []  # (instruction text, wait states it provides)
+    for line in open(asm_path):
+        t = line.strip()
+        if not t or t[0] in ";." or t.endswith(":"):
+            continue
+        op = t.split()[0]
+        if op.startswith("v_mfma"):
+            total += 1
+            ops = [x.strip() for x in t[len(op):].split(",")]
+            src = set().union(*(_regs(o.split()[0]) for o in ops[1:4] if o))
+            waited = 0
+            for h, ws in reversed(hist):
+                if waited >= 2:
+                    break
+                hop = h.split()[0]
+                if hop.startswith("v_") and not hop.startswith(("v_mfma", "v_cmp")):
+                    if _regs(h[len(hop):].split(",")[0].strip()) & src:
+                        bad.append((h, t))
+                waited += ws
+        hist.append((t, int(t.split()[1]) + 1 if op == "s_nop" else 1))
+        if len(hist) > 8:
+            hist.pop(0)
+    return total, bad
+
+
+def check_mfma_hazards(verbose: bool = False) -> int:
+    """Compiles the inline-assembly MFMA kernels to assembly and raises if a hazard is found; returns the MFMA count."""
+    import tempfile
+    flags = [f for f in HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    seen = 0
+    with tempfile.TemporaryDirectory() as tmp:
+        procs = []
+        for src in ASM_MFMA_SOURCES:
+            out = os.path.join(tmp, src + ".s")
+            cmd = [hipcc_path()] + flags + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", out]
+            procs.append((src, out, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        for src, out, cmd, p in procs:
+            log, _ = p.communicate()
+            if p.returncode != 0:
+                raise RuntimeError("hipcc -S failed: %s\n%s" % (" ".join(cmd), log))
+            total, bad = scan_mfma_hazards(out)
+            if verbose:
+                print(f"{src}: {total} MFMAs scanned, {len(bad)} too close to an operand write")
+            if total < 1024:
+                raise RuntimeError(f"{src}: only {total} MFMAs found in the compiler output; the scan is not seeing the kernels")
+            if bad:
+                raise RuntimeError(f"{src}: MFMA operand written fewer than two wait states before the MFMA: {bad[:3]}")
+            seen += total
+    return seen
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv, extra_flags=tuple(a for a in sys.argv[1:] if a.startswith("-D"))))
+    if "--check-hazards" in sys.argv:
+        print(check_mfma_hazards(verbose=True), "MFMAs scanned, no operand hazard")

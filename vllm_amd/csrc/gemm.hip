@@ -140,11 +140,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // ... except that the prefill kernel also has 8-bit (uint8b128, fp8), fp4 and float-zero-point instantiations
   const bool w8 = a->wtype == W4A16_WTYPE_U8B128 || a->wtype == W4A16_WTYPE_FE4M3;
   const bool fat_ok = !general_only || w8 || a->wtype == W4A16_WTYPE_FE2M1 || (a->flags & W4A16_F_ZP_FLOAT);
-  // the 64-row kernel has instantiations for all of them (8-bit MoE weights with act-order are refused just below)
+  // the 64-row kernel has instantiations for all of them
   const bool mid_ok = !general_only || a->wtype == W4A16_WTYPE_FE2M1 || w8 || ((a->flags & W4A16_F_ZP_FLOAT) && !moe);
   const bool pow2_group = (pl.group_ksteps & (pl.group_ksteps - 1)) == 0;  // prefill / 64-row kernels shift
-  if (a->wtype == W4A16_WTYPE_U8B128 && moe && act_order)
-    return fail(W4A16_ENOTIMPL, "8-bit MoE weights with act-order are not implemented in this build");
   if (moe) {
     const int bs = a->moe_block_size;
     pl.mb = bs <= 16 ? 1 : bs <= 32 ? 2 : 4;

@@ -217,14 +217,22 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
 // with v_accvgpr moves (more of them than dequantisation instructions).  Source C == destination is the form
 // the matrix pipe forwards without extra wait states; results are only read again after the main loop.
 // The statement is opaque to the compiler's hazard logic: an operand register must not be written by a VALU
-// instruction in the two wait states before it (callers dequantise operands several MFMAs ahead; a compiler-output
-// test checks the distance).
+// instruction in the two wait states before it.  Callers dequantise every operand register at least one MFMA (16 cycles)
+// ahead of its use and pin that order with scheduling barriers; the build step verifies the compiler's output.
+// (Two wait states in front of every such MFMA, `s_nop 1` inside the statement, would make this unconditional; it costs
+// 5-8 % of the prefill kernels' throughput and is only compiled in with -DW4A16_MFMA_NOP.  The shipped build instead
+// scans its own compiler output for the hazard, see vllm_amd/build.py: check_mfma_hazards.)
+#ifdef W4A16_MFMA_NOP
+#define W4A16_MFMA_PRE "s_nop 1\n\t"
+#else
+#define W4A16_MFMA_PRE ""
+#endif
 template <int DT>
 __device__ __forceinline__ void mfma_inplace(f32x4& acc, const u32x4& a, const u32x4& b) {
   if constexpr (DT == DT_F16)
-    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    asm(W4A16_MFMA_PRE "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   else
-    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    asm(W4A16_MFMA_PRE "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 constexpr int RED_RS = 148;  // row stride (floats) of the 128-column reduction slab (4 mod 16: conflict-free)

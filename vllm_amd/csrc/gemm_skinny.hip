@@ -593,28 +593,32 @@ static skinny_fn pick_mb(int mb, bool zp, int gm) {
   }
 }
 
-template <int DT>
-static skinny_fn pick_w8(int mb, int gm) {  // uint8b128: no zero points, A's columns already in weight order
+template <int DT, bool PERM>
+static skinny_fn pick_w8(int mb, int gm) {  // uint8b128: no zero points; PERM: MoE act-order, A gathered in the kernel
+  if constexpr (PERM) {
+    if (gm == GM_CHANNEL) return nullptr;  // act-order needs groups
+  }
   switch (mb) {
     case 1:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, false, 8>
+      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, PERM, 8>
              : gm == GM_CHANNEL ? skinny_kernel<DT, 1, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 1, false, GM_GIDX, false, 8>;
+                                : skinny_kernel<DT, 1, false, GM_GIDX, PERM, 8>;
     case 2:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, false, 8>
+      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, PERM, 8>
              : gm == GM_CHANNEL ? skinny_kernel<DT, 2, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 2, false, GM_GIDX, false, 8>;
+                                : skinny_kernel<DT, 2, false, GM_GIDX, PERM, 8>;
     default:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, false, 8>
+      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, PERM, 8>
              : gm == GM_CHANNEL ? skinny_kernel<DT, 4, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 4, false, GM_GIDX, false, 8>;
+                                : skinny_kernel<DT, 4, false, GM_GIDX, PERM, 8>;
   }
 }
 
 static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool perm, bool w8) {
   if (w8) {
-    if (zp || perm) return nullptr;
-    return dt == DT_F16 ? pick_w8<DT_F16>(mb, gm) : pick_w8<DT_BF16>(mb, gm);
+    if (zp) return nullptr;
+    if (perm) return dt == DT_F16 ? pick_w8<DT_F16, true>(mb, gm) : pick_w8<DT_BF16, true>(mb, gm);
+    return dt == DT_F16 ? pick_w8<DT_F16, false>(mb, gm) : pick_w8<DT_BF16, false>(mb, gm);
   }
   if (perm) return dt == DT_F16 ? pick_mb<DT_F16, true>(mb, zp, gm) : pick_mb<DT_BF16, true>(mb, zp, gm);
   return dt == DT_F16 ? pick_mb<DT_F16, false>(mb, zp, gm) : pick_mb<DT_BF16, false>(mb, zp, gm);
