@@ -480,11 +480,14 @@ __device__ __forceinline__ float nvfp4_scale_f32(uint32_t byte) {
 // MXFP4 scale byte (E8M0) -> fp32: 2^(b - 127)
 __device__ __forceinline__ float mxfp4_scale_f32(uint32_t byte) { return __builtin_bit_cast(float, byte << 23); }
 
-// "Raw" B operands for the fold scheme of the decode kernel: nibbles are only moved into the mantissa
-// of a magic exponent, value = E + q (E = 1024 for fp16, 128 for bf16) — or, with HI_TRICK (fp16), the
-// high nibbles stay in place: value = 1024 + 16q for the K rows k0+8, k0+9 (slots 1 and 3), which the
-// caller compensates by scaling the matching activations by 1/16.  No subtract, no scale: both are
-// applied to the fp32 accumulator once per quantization group.
+// "Raw" B operands for the fold scheme of the 16-row kernels: nibbles are only moved into the mantissa of a magic
+// exponent, value = E + q (E = 1024 for fp16, 128 for bf16).  With HI_TRICK (fp16) the high nibbles stay where they
+// are, bits 4..7, under the exponent of 64, whose mantissa bits 4..7 weigh 1, 2, 4, 8: value = 64 + q exactly, for the
+// K rows k0+8, k0+9 (slots 1 and 3), so no shift is needed.  No subtract, no scale: both are applied to the fp32
+// accumulator once per quantization group, through a bias-term MFMA whose operand carries 1024 + 8 in the low-nibble
+// slots and 64 + 8 in the high-nibble slots (RAW_BIAS_LO / RAW_BIAS_HI).
+constexpr uint32_t RAW_BIAS_LO = 0x64086408u;  // (1032, 1032)
+constexpr uint32_t RAW_BIAS_HI = 0x54805480u;  // (72, 72)
 template <int DT, bool HI_TRICK>
 __device__ __forceinline__ void raw_pair(uint32_t xa, uint32_t xb, u32x4& o0, u32x4& o1) {
   const uint32_t M = 0x000f000fu;
@@ -492,9 +495,11 @@ __device__ __forceinline__ void raw_pair(uint32_t xa, uint32_t xb, u32x4& o0, u3
   asm("" : "+v"(E));  // keep in a VGPR: (x & mask) | E becomes one v_and_or_b32
   if constexpr (HI_TRICK) {
     const uint32_t MH = 0x00f000f0u;
+    uint32_t EH = 0x54005400u;
+    asm("" : "+v"(EH));
     const uint32_t ya = xa >> 8, yb = xb >> 8;
-    o0 = u32x4{(xa & M) | E, (xa & MH) | E, (xb & M) | E, (xb & MH) | E};
-    o1 = u32x4{(ya & M) | E, (ya & MH) | E, (yb & M) | E, (yb & MH) | E};
+    o0 = u32x4{(xa & M) | E, (xa & MH) | EH, (xb & M) | E, (xb & MH) | EH};
+    o1 = u32x4{(ya & M) | E, (ya & MH) | EH, (yb & M) | E, (yb & MH) | EH};
   } else {
     o0 = u32x4{(xa & M) | E, ((xa >> 4) & M) | E, (xb & M) | E, ((xb >> 4) & M) | E};
     o1 = u32x4{((xa >> 8) & M) | E, ((xa >> 12) & M) | E, ((xb >> 8) & M) | E, ((xb >> 12) & M) | E};

@@ -10,7 +10,7 @@
 //   * a pipeline stage is two k-steps (64 K rows): 4 weight loads, 2 activation loads that read 128
 //     contiguous bytes per row (full cache lines), one scale load, one zero-point load.
 //   * "fold" arithmetic: nibbles are only OR-ed into the mantissa of a magic exponent (fp16: 1024+q or, for
-//     the high nibbles, 1024+16q against activations pre-scaled by 1/16; bf16: 128+q) and fed to the MFMA as
+//     the high nibbles, which stay at bits 4..7, 64+q; bf16: 128+q) and fed to the MFMA as
 //     they are; one extra MFMA per k-step against a constant operand accumulates the bias term
 //     sum_k a_k * (E+8)  [or sum_k a_k when zero points vary per column].  Once per quantization group the fp32
 //     partial is folded:  acc += s * (tmp - (E+z) * rs).  Exact integer dequantisation happens in fp32, the
@@ -164,13 +164,15 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
         s.a[i] = *(const u32x4*)(arow[i] + sidx * 64);
       }
     }
-    const int gi = CHANNEL ? 0 : (2 * sidx) / p.group_ksteps;
+    // (channel-wise scales: fold every 128 K rows all the same, so that the raw partial sums, biased by E * sum(a),
+    //  stay small next to fp32's 24 bits whatever the activations' mean)
+    const int gi = CHANNEL ? (sidx >> 1) : (p.group_shift >= 0 ? (2 * sidx) >> p.group_shift : (2 * sidx) / p.group_ksteps);
     s.gi = gi;
     if (!CHANNEL)
       s.sc = *(const bvec*)(sp + (int64_t)gi * p.N);
     else
       s.sc = bvec(0);
-    if (ZP) s.zq = zp[(int64_t)gi * (p.N >> 3)];
+    if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (p.N >> 3)];
     const uint32_t* q = bp + (int64_t)(4 * (sidx - w_b)) * b_row;
 #pragma unroll
     for (int t = 0; t < 4; ++t) s.b[t] = __builtin_nontemporal_load((const bvec*)(q + t * b_row));
@@ -238,13 +240,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     }
     u32x4 vb;  // B operand of the bias-term MFMA
     if constexpr (HI_TRICK) {
-      const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        af[kk][1] = as_u32(as_h2(af[kk][1]) * sixteenth);
-        af[kk][3] = as_u32(as_h2(af[kk][3]) * sixteenth);
-      }
-      vb = u32x4{0x64086408u, 0x64806480u, 0x64086408u, 0x64806480u};  // 1032 | 1152 = 16 * 72
+      vb = u32x4{RAW_BIAS_LO, RAW_BIAS_HI, RAW_BIAS_LO, RAW_BIAS_HI};
     } else {
       const uint32_t one = (DT == DT_F16) ? 0x3c003c00u : 0x3f803f80u;
       vb = u32x4{one, one, one, one};

@@ -198,13 +198,16 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     int gi = 0;
     s.uni = true;
     if (GM == GM_GROUPED) gi = ks / p.group_ksteps;
+    // channel-wise scales on the fold path: fold every 128 K rows all the same, so that the raw partial sums (biased
+    // by E * sum(a)) stay small next to fp32's 24 bits whatever the activations' mean
+    if (FOLD && GM == GM_CHANNEL) gi = ks >> 2;
     if (GM == GM_GIDX) {
       gi = gidx[ks * 32];
       s.uni = (gidx[ks * 32 + 31] == gi);
     }
     s.gi = gi;
     if (GM != GM_CHANNEL) s.sc = sp[(int64_t)gi * s_row];
-    if (ZP) s.zq = zp[(int64_t)gi * s_row];
+    if (ZP) s.zq = zp[(int64_t)(GM == GM_CHANNEL ? 0 : gi) * s_row];
     if (ZPF) s.zf = zfp[(int64_t)gi * s_row];
     if (FP4 == 2) s.zq = ks & 1;  // which half of the two-k-step scale record
     s.b0 = __builtin_nontemporal_load(bp + (int64_t)(2 * ks) * b_row);
@@ -322,11 +325,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       }
       u32x4 vb;  // B operand of the bias-term MFMA
       if constexpr (HI_TRICK) {
-        // activations of the high-nibble K rows (slots 1, 3) are scaled by 1/16 (exact)
-        const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-        af[0][1] = as_u32(as_h2(af[0][1]) * sixteenth);
-        af[0][3] = as_u32(as_h2(af[0][3]) * sixteenth);
-        vb = u32x4{0x64086408u, 0x64806480u, 0x64086408u, 0x64806480u};  // 1032, 1152 = 16 * 72
+        vb = u32x4{RAW_BIAS_LO, RAW_BIAS_HI, RAW_BIAS_LO, RAW_BIAS_HI};
       } else {
         const uint32_t one = (DT == DT_F16) ? 0x3c003c00u : 0x3f803f80u;
         vb = u32x4{one, one, one, one};
