@@ -27,11 +27,21 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0
 LAYERS = {"qkv": (4096, 6144), "o": (4096, 4096), "gate_up": (4096, 28672), "down": (14336, 4096)}
 GROUP = 128
-# HBM bytes per launch of the headline step's GEMM kernel (average of the four launches at M=16), from two
-# `rocprofv3 --pmc` runs of `bench.py --pmc-probe` (FETCH_SIZE, WRITE_SIZE), each scaled by what the same
-# counter reads for the 256 MiB device copy in that run (FETCH_SIZE reads 0.5 per KiB copied, WRITE_SIZE 1.0):
-# read + written KiB: qkv 14647 + 966, o 10657 + 1160, gate_up 60419 + 896, down 34400 + 1160.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = (14647 + 966 + 10657 + 1160 + 60419 + 896 + 34400 + 1160) * 1024 / 4
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "decode_kernel_llama3_8b_M16_hbm_traffic_pmc.txt")
+
+
+def measured_traffic_bytes_per_launch():
+    """HBM bytes per launch of the headline step's GEMM kernel (average of the four launches at M = 16) as the counter
+    summary under profiles/ states it (`traffic_bytes_per_launch = N`, from FETCH_SIZE and WRITE_SIZE scaled by a copy of
+    known size); None when the summary is missing or carries no such line."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("traffic_bytes_per_launch"):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def algorithmic_bytes(m, k, n, zp=False, act_order=False):
@@ -166,6 +176,34 @@ def bench_repack(ops, dev):
                                      "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS}
             print(f"[detail] {kind} repack {name}: {sec * 1e6:.1f} us, {by / sec / 1e9:.0f} GB/s = "
                   f"{100 * by / sec / 1e9 / HBM_PEAK_GBPS:.1f}% HBM", file=sys.stderr, flush=True)
+    return out
+
+
+def bench_load_path(ops, dev):
+    """Load-time preparation of one Llama-3-8B decoder layer's four linears from checkpoint tensors (AWQ layout: packed
+    weights, packed zero points, scales): repack + scale permutation + zero-point conversion, all on the device; bytes =
+    checkpoint bytes read + Marlin bytes written.  Also projected to the 32 layers of the model."""
+    from vllm_amd.marlin_utils import awq_to_marlin_zero_points, marlin_permute_scales
+    layers = []
+    for name, (k, n) in LAYERS.items():
+        g = torch.Generator(device=dev).manual_seed(11)
+        qw = torch.randint(-2**31, 2**31 - 1, (k, n // 8), generator=g, device=dev, dtype=torch.int32)
+        qz = torch.randint(-2**31, 2**31 - 1, (k // GROUP, n // 8), generator=g, device=dev, dtype=torch.int32)
+        sc = torch.rand(k // GROUP, n, generator=g, device=dev).to(torch.bfloat16)
+        layers.append((k, n, qw, qz, sc))
+
+    def prepare():
+        for k, n, qw, qz, sc in layers:
+            ops.awq_marlin_repack(qw, k, n, 4)
+            marlin_permute_scales(sc, k, n, GROUP)
+            awq_to_marlin_zero_points(qz, k // GROUP, n, 4)
+    sec = time_graph([prepare], reps=5, warmup=1)
+    by = sum(2 * (qw.numel() * 4 + qz.numel() * 4 + sc.numel() * 2) for _, _, qw, qz, sc in layers)
+    out = {"us_per_decoder_layer": sec * 1e6, "GBps": by / sec / 1e9, "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS,
+           "launches_per_decoder_layer": 12, "ms_for_32_layers": 32 * sec * 1e3}
+    print(f"[detail] load path, one decoder layer (4 linears, AWQ checkpoint -> Marlin operands): {sec * 1e6:.1f} us, "
+          f"{by / sec / 1e9:.0f} GB/s = {100 * out['hbm_frac']:.1f}% HBM; 32 layers: {32 * sec * 1e3:.2f} ms",
+          file=sys.stderr, flush=True)
     return out
 
 
@@ -354,6 +392,12 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection workload: plain device copies of known size (calibration) followed by "
                          "eager launches of the headline GEMMs on cold weights; prints no JSON line")
+    ap.add_argument("--probe-shape", type=str, default="",
+                    help="counter-collection workload for one shape, LAYER:M:KIND with KIND gptq_f16 or awq_bf16 "
+                         "(e.g. gate_up:4096:awq_bf16): a few eager launches on rotating weight copies; prints no JSON line")
+    ap.add_argument("--issue-probe", action="store_true",
+                    help="MFMA / VALU issue micro-benchmark (independent MFMAs interleaved with 0..6 VALU instructions, "
+                         "one and two wavefronts per SIMD); prints a table, no JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1", file=sys.stderr)
@@ -369,6 +413,26 @@ def main():
     torch.cuda.set_device(dev)
     workspace = marlin_make_workspace_new(dev)
     m = args.m
+
+    if args.issue_probe:
+        from vllm_amd import issue_probe
+        issue_probe.run(dev)
+        return
+    if args.probe_shape:
+        name, pm, kind = args.probe_shape.split(":")
+        k, n = LAYERS[name]
+        if kind == "awq_bf16":
+            base, wt, dt = make_awq_layer(ops, k, n, torch.bfloat16, dev, 1), scalar_types.uint4, torch.bfloat16
+        else:
+            base, wt, dt = make_gptq_layer(ops, k, n, torch.float16, dev, 1), scalar_types.uint4b8, torch.float16
+        ncopy = min(copies_needed(base["q"].numel() * 4), 16)
+        copies = [base] + [clone_weights(base, 100 + i) for i in range(ncopy - 1)]
+        a = torch.randn(int(pm), k, generator=torch.Generator().manual_seed(2)).to(dt).to(dev)
+        for i in range(2 * ncopy):
+            gemm(ops, wt, a, copies[i % ncopy], workspace)
+        torch.cuda.synchronize()
+        print(f"probe-shape done: {2 * ncopy} launches of {name} M={pm} {kind}", file=sys.stderr)
+        return
 
     # ---- headline: one step = the four decode GEMMs, weights rotated over `nsets` full sets
     step_wbytes = sum(k * n // 2 for k, n in LAYERS.values())
@@ -454,7 +518,7 @@ def main():
                    "shapes_KN": list(LAYERS.values()), "M": m, "weight_sets_rotated": nsets,
                    "timing": "HIP graph replay between two events on the launch stream"},
         "roofline": {"bound": "hbm", "achieved": step_bytes / 4 / avg_launch_s / 1e9, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": step_bytes / 4 / avg_launch_s / 1e9 / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if m == 16 else None,
+                     "unit": "GB/s", "frac": step_bytes / 4 / avg_launch_s / 1e9 / HBM_PEAK_GBPS, "traffic": measured_traffic_bytes_per_launch() if m == 16 else None,
                      "kernel": "w4a16::decode_kernel<f16, no-zp, grouped> (64- and 128-column instantiations, "
                                "average over the step's four launches)", "launches": launches,
                      "avg_launch_us": avg_launch_s * 1e6, "algorithmic_bytes_per_launch": step_bytes / 4},
@@ -485,6 +549,7 @@ def main():
         detail["mixtral_moe_fp16_gptq"] = bench_moe(ops, scalar_types.uint4b8, dev)
         torch.cuda.empty_cache()
         detail["repack"] = bench_repack(ops, dev)
+        detail["load_path"] = bench_load_path(ops, dev)
         torch.cuda.empty_cache()
         detail["other_weight_types_gate_up_warm"] = bench_other_types(ops, dev, workspace)
         result["detail"] = detail
@@ -494,6 +559,19 @@ def main():
             "prefill_bf16_awq_us": {k: round(v["us"], 1) for k, v in detail["prefill_bf16_awq"].items()},
             "prefill_bf16_awq_mfma_frac": {k: round(v["mfma_frac"], 3) for k, v in detail["prefill_bf16_awq"].items()},
         }
+        # the M = 4096 half of the metric: the prefill kernel on the four bf16 AWQ layers, against the dense MFMA peak
+        pf = detail["prefill_bf16_awq"]
+        pf_flops = sum(2.0 * v["m"] * v["n"] * v["k"] for v in pf.values())
+        pf_sec = sum(v["us"] for v in pf.values()) * 1e-6
+        result["roofline_mfma"] = {
+            "bound": "mfma", "achieved": pf_flops / pf_sec / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": pf_flops / pf_sec / 1e12 / MFMA_PEAK_TFLOPS, "traffic": None,
+            "kernel": "w4a16::fat_kernel<bf16, zero points, grouped> (qkv also runs its last 512-column strips on "
+                      "w4a16::mid_kernel)", "launches": sum(v["launches_timed"] for v in pf.values()),
+            "flops_per_launch_avg": pf_flops / 4, "avg_launch_us": pf_sec / 4 * 1e6,
+            "workload": "llama3-8b linears at M=4096, bf16, AWQ uint4 + uint4 zero points g128 (qkv, o, gate_up, down), "
+                        "time-weighted over the four layers",
+            "per_layer_frac": {k: round(v["mfma_frac"], 3) for k, v in pf.items()}}
         if args.table:
             with open(args.table, "w") as f:
                 json.dump(detail, f, indent=1)

@@ -53,7 +53,19 @@ def build(verbose: bool = False, extra_flags: tuple = ()) -> str:
     if r.returncode != 0:
         raise RuntimeError("link failed: %s\n%s" % (" ".join(cmd), r.stdout))
     os.replace(tmp, LIB_PATH)
+    build_probe()
     return LIB_PATH
+
+
+def build_probe() -> str:
+    """The MFMA / VALU issue micro-benchmark of `bench.py --issue-probe`: a library of its own, not linked into the product."""
+    out = os.path.join(HERE, "libw4a16_probe.so")
+    cmd = [hipcc_path()] + HIPCC_FLAGS + [os.path.join(CSRC, "issue_probe.hip"), "-o", out + ".tmp"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), r.stdout))
+    os.replace(out + ".tmp", out)
+    return out
 
 
 # ---------------------------------------------------------------------------------------------------------------
