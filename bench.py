@@ -398,6 +398,9 @@ def main():
     ap.add_argument("--issue-probe", action="store_true",
                     help="MFMA / VALU issue micro-benchmark (independent MFMAs interleaved with 0..6 VALU instructions, "
                          "one and two wavefronts per SIMD); prints a table, no JSON line")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="streaming floor of the 16-row kernels on the four layers (a kernel with their loads and no "
+                         "arithmetic); prints a table, no JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1", file=sys.stderr)
@@ -417,6 +420,10 @@ def main():
     if args.issue_probe:
         from vllm_amd import issue_probe
         issue_probe.run(dev)
+        return
+    if args.stream_probe:
+        from vllm_amd import issue_probe
+        issue_probe.stream_floor(dev, LAYERS, time_graph, copies_needed)
         return
     if args.probe_shape:
         name, pm, kind = args.probe_shape.split(":")

@@ -141,6 +141,13 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   uint32_t* slab_wr = slab + ar * A_ROW + ap * 4;
   const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
 
+  // rows 8..15 of the tile exist?  (otherwise their activation loads are skipped)
+  const bool rows_hi = p.moe ? (p.moe_bs > 8) : (mt * 16 + 8 < p.M);
+  // scale group of an absolute stage index (channel-wise scales: pseudo-groups of 128 K rows, so that the raw partial
+  // sums, biased by E * sum(a), stay small next to fp32's 24 bits whatever the activations' mean)
+  auto group_of = [&](int sidx) {
+    return CHANNEL ? (sidx >> 1) : (p.group_shift >= 0 ? (2 * sidx) >> p.group_shift : (2 * sidx) / p.group_ksteps);
+  };
   struct Stage {
     bvec b[4];   // k-tiles 4s .. 4s+3
     u32x4 a[2];  // rows ar, ar+8
@@ -160,19 +167,18 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
         for (int j = 0; j < 8; ++j) e[j] = row[perm[sidx * 64 + ap * 8 + j]];
         s.a[i] = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
                        (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+      } else if (i == 1 && !rows_hi) {
+        s.a[i] = u32x4{0, 0, 0, 0};  // the tile has no rows 8..15
       } else {
         s.a[i] = *(const u32x4*)(arow[i] + sidx * 64);
       }
     }
-    // (channel-wise scales: fold every 128 K rows all the same, so that the raw partial sums, biased by E * sum(a),
-    //  stay small next to fp32's 24 bits whatever the activations' mean)
-    const int gi = CHANNEL ? (sidx >> 1) : (p.group_shift >= 0 ? (2 * sidx) >> p.group_shift : (2 * sidx) / p.group_ksteps);
+    const int gi = group_of(sidx);
     s.gi = gi;
-    if (!CHANNEL)
-      s.sc = *(const bvec*)(sp + (int64_t)gi * p.N);
-    else
-      s.sc = bvec(0);
-    if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (p.N >> 3)];
+    if (sidx == w_b || gi != group_of(sidx - 1)) {  // uniform: only the first stage of a group carries its scales
+      if (!CHANNEL) s.sc = *(const bvec*)(sp + (int64_t)gi * p.N);
+      if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (p.N >> 3)];
+    }
     const uint32_t* q = bp + (int64_t)(4 * (sidx - w_b)) * b_row;
 #pragma unroll
     for (int t = 0; t < 4; ++t) s.b[t] = __builtin_nontemporal_load((const bvec*)(q + t * b_row));

@@ -88,3 +88,69 @@ extern "C" float w4a16_issue_probe(const uint32_t* in, float* out, int workgroup
   hipEventDestroy(e1);
   return best;
 }
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// Streaming floor of the 16-row GEMM kernels: the same work decomposition and access pattern as decode_kernel (one
+// workgroup of 8 wavefronts per TN-column tile and K split, wavefronts cut the K range into contiguous parts, DEPTH
+// stages of four k-tile loads in flight per wavefront, 16 or 8 bytes per lane and load, non-temporal) but nothing is
+// computed: the words are xor-ed together and never stored.  What this takes is what a GEMM kernel of this shape cannot
+// beat on the part.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <int TN, int DEPTH>
+__global__ __launch_bounds__(512) void stream_probe_kernel(const uint32_t* __restrict__ w, uint32_t* __restrict__ sink,
+                                                           int K, int N, int splits) {
+  using vec = uint32_t __attribute__((ext_vector_type(TN / 32)));
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
+  const int nsp = splits < 0 ? -splits : splits;
+  const int tile = blockIdx.x / nsp, split = blockIdx.x % nsp;
+  const int stages = K / 64;  // a stage = four k-tiles = 64 K rows
+  const int per_split = (stages + nsp - 1) / nsp;
+  const int st_b = split * per_split, st_e = min(st_b + per_split, stages);
+  const int per = (st_e - st_b + 7) / 8;
+  const int w_b = min(st_b + wv * per, st_e), w_e = min(w_b + per, st_e);
+  const int nt = TN == 128 ? 2 * tile + h : tile;
+  const int64_t row = (int64_t)N * 2;
+  const uint32_t* p = w + (int64_t)nt * 128 + (4 * c + g) * 4 + (TN == 64 ? 2 * h : 0) + (int64_t)(4 * w_b) * row;
+  vec acc = vec(0);
+  vec st[DEPTH][4];
+  const int n = w_e - w_b;
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j)
+    if (j < n)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) st[j][t] = __builtin_nontemporal_load((const vec*)(p + (int64_t)(4 * j + t) * row));
+  for (int i = 0; i < n; i += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+      if (i + j < n) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc ^= st[j][t];
+        if (i + j + DEPTH < n)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            st[j][t] = __builtin_nontemporal_load((const vec*)(p + (int64_t)(4 * (i + j + DEPTH) + t) * row));
+      }
+    }
+  }
+  uint32_t x = 0;
+#pragma unroll
+  for (int t = 0; t < TN / 32; ++t) x ^= acc[t];
+  if (splits < 0) sink[(size_t)blockIdx.x * 512 + threadIdx.x] = x;  // (negative split count: also write 2 KB per workgroup)
+  else if (x == 0x12345678u) sink[threadIdx.x] = x;
+}
+
+// w: int32 [K/16, 2N] (any contents); sink: >= 512 dwords, or, with a negative split count (same split, but every
+// workgroup also stores 2 KB), >= 512 dwords per workgroup.  Launches on `stream`; returns 0 or a negative code.
+extern "C" int w4a16_stream_probe(const uint32_t* w, uint32_t* sink, int K, int N, int tn, int splits, int depth,
+                                  void* stream) {
+  if (K % 64 || N % 128 || splits == 0 || (tn != 64 && tn != 128) || (depth != 3 && depth != 6)) return -1;
+  const int grid = (N / tn) * (splits < 0 ? -splits : splits);
+  hipStream_t s = (hipStream_t)stream;
+  if (tn == 128 && depth == 3) hipLaunchKernelGGL((stream_probe_kernel<128, 3>), dim3(grid), dim3(512), 0, s, w, sink, K, N, splits);
+  if (tn == 128 && depth == 6) hipLaunchKernelGGL((stream_probe_kernel<128, 6>), dim3(grid), dim3(512), 0, s, w, sink, K, N, splits);
+  if (tn == 64 && depth == 3) hipLaunchKernelGGL((stream_probe_kernel<64, 3>), dim3(grid), dim3(512), 0, s, w, sink, K, N, splits);
+  if (tn == 64 && depth == 6) hipLaunchKernelGGL((stream_probe_kernel<64, 6>), dim3(grid), dim3(512), 0, s, w, sink, K, N, splits);
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}

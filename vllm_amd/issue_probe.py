@@ -41,3 +41,54 @@ def run(dev, iters: int = 2000) -> list[dict]:
                     print(f"{data:6s} waves/SIMD={waves // 4} VALU/MFMA={nv} {'chained' if dep else 'independent'}: "
                           f"{per_simd_ns:6.2f} ns per MFMA and SIMD, {tflops:7.0f} TFLOP/s", flush=True)
     return rows
+
+
+def stream_floor(dev, layers: dict, time_graph, copies_needed) -> dict:
+    """Streaming floor of the 16-row GEMM kernels (`bench.py --stream-probe`): a kernel with decode_kernel's work
+    decomposition and loads that computes nothing, on weight buffers not touched for >= 512 MB of other traffic, replayed
+    from a HIP graph like the GEMM rows of the bench table.  Per layer the best of the launch shapes the planner can
+    choose from (tile width 64 / 128, K splits that keep the grid within one workgroup per compute unit, 3 or 6 stages in
+    flight)."""
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.w4a16_stream_probe.restype = ctypes.c_int
+    lib.w4a16_stream_probe.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.zeros(512, dtype=torch.int32, device=dev)
+    out = {}
+    for name, (k, n) in layers.items():
+        nbytes = k * n // 2
+        ncopy = copies_needed(nbytes)
+        bufs = [torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev) for _ in range(ncopy)]
+        best = None
+        for tn in (128, 64):
+            for splits in (1, 2, 3, 4, 6, 8):
+                if splits > 1 and (n // tn) * splits > cus:
+                    continue
+                if k // 64 // splits < 8:
+                    continue
+                for depth in (3, 6):
+                    def launch(b):
+                        rc = lib.w4a16_stream_probe(b.data_ptr(), sink.data_ptr(), k, n, tn, splits, depth,
+                                                    torch.cuda.current_stream(dev).cuda_stream)
+                        assert rc == 0, rc
+                    fns = [(lambda b=bufs[i % ncopy]: launch(b)) for i in range(max(40, ncopy))]
+                    us = time_graph(fns, reps=3, warmup=1) / len(fns) * 1e6
+                    if best is None or us < best["us"]:
+                        best = dict(us=us, tile_columns=tn, k_splits=splits, stages_in_flight=depth,
+                                    GBps=nbytes / us / 1e3)
+        # the same launch shape with every workgroup also storing 2 KB: what it costs a kernel to write at all
+        big_sink = torch.zeros((n // best["tile_columns"]) * best["k_splits"] * 512, dtype=torch.int32, device=dev)
+
+        def launch_w(b):
+            rc = lib.w4a16_stream_probe(b.data_ptr(), big_sink.data_ptr(), k, n, best["tile_columns"], -best["k_splits"],
+                                        best["stages_in_flight"], torch.cuda.current_stream(dev).cuda_stream)
+            assert rc == 0, rc
+        fns = [(lambda b=bufs[i % ncopy]: launch_w(b)) for i in range(max(40, ncopy))]
+        best["us_with_stores"] = time_graph(fns, reps=3, warmup=1) / len(fns) * 1e6
+        out[name] = best
+        print(f"stream floor {name} ({k} x {n}, {nbytes / 1e6:.1f} MB): {best['us']:.2f} us = {best['GBps']:.0f} GB/s "
+              f"(tiles of {best['tile_columns']} columns, {best['k_splits']} K splits, {best['stages_in_flight']} stages in "
+              f"flight); {best['us_with_stores']:.2f} us when every workgroup also stores 2 KB", flush=True)
+        del bufs
+        torch.cuda.empty_cache()
+    return out
