@@ -17,7 +17,8 @@ What it does, in order:
      csrc/torch_bindings.cpp:240, csrc/moe/torch_bindings.cpp:52);
   2. puts `Gfx950MarlinLinearKernel` in front of `_POSSIBLE_KERNELS`
      (vllm/model_executor/layers/quantization/kernels/mixed_precision/__init__.py:36-45), so `choose_mp_linear_kernel`
-     finds a kernel for uint4b8 / uint8b128 / uint4 + zero points on this platform;
+     finds a kernel for uint4b8 / uint8b128 / uint4 + zero points on this platform; the class is vLLM's own
+     MarlinLinearKernel with `can_implement` replaced (see `register_kernel_class`);
   3. lifts the CUDA-only gates in front of the Marlin quantization configs: `is_gptq_marlin_compatible`
      (gptq_marlin.py:254-279), `is_awq_marlin_compatible` (awq_marlin.py:216-241) and the ROCm platform's
      `supported_quantization` list (platforms/rocm.py:175-187).
@@ -43,19 +44,33 @@ def _try_import(name: str):
         return None
 
 
-def register_kernel_class() -> bool:
-    """Step 2: a subclass of this library's MarlinLinearKernel, under a name of its own so that vLLM's
-    VLLM_DISABLED_KERNELS=MarlinLinearKernel still only addresses vLLM's CUDA kernel."""
+def register_kernel_class(own_load_path: bool = False) -> bool:
+    """Step 2.  The class put in front of `_POSSIBLE_KERNELS` is named Gfx950MarlinLinearKernel, so that vLLM's
+    VLLM_DISABLED_KERNELS=MarlinLinearKernel still only addresses vLLM's CUDA kernel.
+
+    With vLLM's own `MarlinLinearKernel` importable (kernels/mixed_precision/marlin.py:27) the class derives from
+    THAT one and overrides `can_implement` alone (marlin.py:33-59, whose first test is "CUDA only"): weight
+    preparation and `apply_weights` stay vLLM's code, which reaches this library through the `_C` operators of
+    step 1, so parameter handling follows the installed vLLM version.  `own_load_path=True`, or a vLLM without that
+    module, registers this library's class instead, which prepares a layer with its device-side kernels
+    (`vllm_amd.mixed_precision.prepare_marlin_layer`)."""
     mp = _try_import(_MP_KERNELS)
     if mp is None or not hasattr(mp, "_POSSIBLE_KERNELS"):
         return False
-    from .mixed_precision import MarlinLinearKernel
+    from .mixed_precision import MarlinLinearKernel as OwnKernel
 
     if any(k.__name__ == "Gfx950MarlinLinearKernel" for k in mp._POSSIBLE_KERNELS):
         return True
 
-    class Gfx950MarlinLinearKernel(MarlinLinearKernel):
-        pass
+    theirs = None if own_load_path else getattr(_try_import(_MP_KERNELS + ".marlin"), "MarlinLinearKernel", None)
+    if theirs is not None:
+        class Gfx950MarlinLinearKernel(theirs):
+            @classmethod
+            def can_implement(cls, c):
+                return OwnKernel.can_implement(c)   # the reference's rule without its platform test
+    else:
+        class Gfx950MarlinLinearKernel(OwnKernel):
+            pass
 
     mp._POSSIBLE_KERNELS.insert(0, Gfx950MarlinLinearKernel)
     return True
