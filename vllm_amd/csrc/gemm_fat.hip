@@ -197,6 +197,32 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     u32x4 af[FB_MB];
 #pragma unroll
     for (int mb = 0; mb < FB_MB; ++mb) af[mb] = abase[mb * 64];
+    // bf16 integer weights: the three dependent stages of one operand register (nibbles -> two floats, two fmas,
+    // one pack) are spread over three consecutive MFMA pairs, so that no VALU instruction reads the result of the
+    // one issued just before it
+    constexpr bool PIPE = (BITS == 4 && FP4 == 0 && !ZPF && DT == DT_BF16);
+    float pc0 = 0.f, pc1 = 0.f, pf0 = 0.f, pf1 = 0.f;
+    auto stage_a = [&](auto p_tag) {  // piece P: nibble bytes -> floats
+      constexpr int P = decltype(p_tag)::value, w = P >> 3, J = P & 7, HF = J >> 2, Q = J & 3;
+      const uint32_t x = (Q < 2) ? nxt.b0[w] : nxt.b1[w];
+      const uint32_t m = ((Q & 1) ? (x >> 4) : x) & 0x0f0f0f0fu;
+      pc0 = ubyte_f32<HF>(m);
+      pc1 = ubyte_f32<HF + 2>(m);
+    };
+    auto stage_b = [&](auto p_tag) {  // (q - z) * s in fp32, exact
+      constexpr int P = decltype(p_tag)::value, w = P >> 3, HF = (P & 7) >> 2;
+      const ColConst<DT> cc = col_const(nxt, w);
+      if constexpr (DT == DT_BF16) {
+        const float sf = HF ? cc.s1 : cc.s0, cf = HF ? cc.c1 : cc.c0;
+        pf0 = __builtin_fmaf(pc0, sf, cf);
+        pf1 = __builtin_fmaf(pc1, sf, cf);
+      }
+    };
+    if constexpr (PIPE) {
+      stage_a(std::integral_constant<int, 0>{});
+      stage_b(std::integral_constant<int, 0>{});
+      stage_a(std::integral_constant<int, 1>{});
+    }
     auto word = [&](auto w_tag) {
       constexpr int w = decltype(w_tag)::value;
       const ColConst<DT> cc = col_const(nxt, w);
@@ -209,7 +235,12 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
         mfma_inplace<DT>(acc[J][w][0], af[J], ob[CUR][w][0]);
         mfma_inplace<DT>(acc[J][w][1], af[J], ob[CUR][w][1]);
         uint32_t r;
-        if constexpr (ZPF)
+        if constexpr (PIPE) {
+          constexpr int P = 8 * w + J;
+          r = pack_bf16(pf0, pf1);
+          if constexpr (P + 1 < 32) stage_b(std::integral_constant<int, P + 1>{});
+          if constexpr (P + 2 < 32) stage_a(std::integral_constant<int, P + 2>{});
+        } else if constexpr (ZPF)
           r = dequant_piece_zpf<J>(xa, xb, nxt.sc[w], zs);
         else if constexpr (FP4 != 0)
           r = ((J & 3) < 2) ? dequant_piece_fp4<DT, J>(xa, fs.a0, fs.a1) : dequant_piece_fp4<DT, J>(xb, fs.b0, fs.b1);
