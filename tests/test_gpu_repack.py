@@ -66,11 +66,18 @@ def test_repack_full_size_roundtrip(ops, dev):
 def test_permute_cols(ops, dev):
     """y == x[:, perm] (reference tests/kernels/core/test_permute_cols.py), including a strided view."""
     g = torch.Generator().manual_seed(1)
-    for m, k in [(1, 128), (33, 4096), (512, 14336)]:
-        x = torch.randn(m, k + 64, generator=g).half().to(dev)[:, :k]
+    # (rows, columns, extra row stride): both kernels behind the op (element-wise for few rows or short / odd rows, rows
+    # staged in LDS otherwise), rows shared between workgroups (32..127 rows), several rows per workgroup (> 1024 rows),
+    # the longest row the staged kernel takes and the first one it does not
+    for m, k, pad in [(1, 128, 64), (33, 4096, 64), (31, 4096, 0), (100, 1024, 8), (512, 14336, 64), (1500, 2048, 0),
+                      (40, 32768, 0), (40, 32776, 0), (64, 1028, 4), (300, 4096, 4)]:
+        x = torch.randn(m, k + pad, generator=g).half().to(dev)[:, :k]
         perm = torch.randperm(k, generator=g).to(torch.int32).to(dev)
         y = ops.permute_cols(x, perm)
-        assert torch.equal(y, x[:, perm.long()])
+        assert torch.equal(y, x[:, perm.long()]), (m, k, pad)
+    x = torch.randn(200, 2048, generator=g).to(torch.bfloat16).to(dev)
+    perm = torch.randperm(2048, generator=g).to(torch.int32).to(dev)
+    assert torch.equal(ops.permute_cols(x, perm), x[:, perm.long()])
 
 
 def test_repack_errors(ops, dev):
