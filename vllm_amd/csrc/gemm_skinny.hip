@@ -352,36 +352,51 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       }
       return;
     }
-    if (GM == GM_GIDX && !s.uni) {
-      // group boundary inside the k-step: fetch the scale row of every K-row separately
+    if constexpr (GM == GM_GIDX) {
+      // Per-row scale lookup.  A k-step inside one group dequantises with the stage's scale row like the grouped form;
+      // one that crosses a group boundary dequantises without a scale and multiplies every operand register (two K rows
+      // of one column) by its own scale pair, fetched as word w of the scale rows of the lane's eight K rows (eight 4-byte
+      // loads per Marlin word, cache hits).  The two forms only differ in how the eight operand registers of a word are
+      // made; the MFMAs follow the merge, so the 32 * MB accumulators are not merged from two branches.
       const int kb = ks * 32 + 2 * g;
-      u32x4 se[8];
+      int64_t srow[8];
+      if (!s.uni) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int kk = kb + (e & 1) + ((e >> 1) & 1) * 8 + (e >> 2) * 16;
-        se[e] = sp[(int64_t)gidx[kk] * s_row];
+        for (int e = 0; e < 8; ++e) {
+          const int kk = kb + (e & 1) + ((e >> 1) & 1) * 8 + (e >> 2) * 16;
+          srow[e] = (int64_t)gidx[kk] * s_row;
+        }
       }
       auto gidx_word = [&](auto w_tag) {
         constexpr int w = decltype(w_tag)::value;
-        u32x4 o[2];
-        dequant_word(s, w_tag, std::true_type{}, o[0], o[1]);
+        u32x4 r[2];
+        if (s.uni) {
+          dequant_word(s, w_tag, std::false_type{}, r[0], r[1]);
+        } else {
+          uint32_t se[8];
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          u32x4 r;
+          for (int e = 0; e < 8; ++e) se[e] = ((const uint32_t*)(sp + srow[e]))[w];
+          u32x4 o[2];
+          dequant_word(s, w_tag, std::true_type{}, o[0], o[1]);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint32_t sa = (se[2 * q][w] >> (16 * hf)) & 0xffffu;
-            const uint32_t sb = (se[2 * q + 1][w] >> (16 * hf)) & 0xffffu;
-            const uint32_t spair = sa | (sb << 16);
-            if constexpr (DT == DT_F16)
-              r[q] = as_u32(as_h2(o[hf][q]) * as_h2(spair));
-            else
-              r[q] = pack_bf16(bf16_lo_f32(o[hf][q]) * bf16_lo_f32(spair),
-                               bf16_hi_f32(o[hf][q]) * bf16_hi_f32(spair));
+          for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t sa = (se[2 * q] >> (16 * hf)) & 0xffffu;
+              const uint32_t sb = (se[2 * q + 1] >> (16 * hf)) & 0xffffu;
+              const uint32_t spair = sa | (sb << 16);
+              if constexpr (DT == DT_F16)
+                r[hf][q] = as_u32(as_h2(o[hf][q]) * as_h2(spair));
+              else
+                r[hf][q] = pack_bf16(bf16_lo_f32(o[hf][q]) * bf16_lo_f32(spair),
+                                     bf16_hi_f32(o[hf][q]) * bf16_hi_f32(spair));
+            }
           }
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb) acc[mb][w][hf] = mfma16x16x32<DT>(af[mb], r, acc[mb][w][hf]);
         }
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[mb][w][hf] = mfma16x16x32<DT>(af[mb], r[hf], acc[mb][w][hf]);
       };
       gidx_word(std::integral_constant<int, 0>{});
       gidx_word(std::integral_constant<int, 1>{});
