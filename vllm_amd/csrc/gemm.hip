@@ -166,9 +166,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
 
   // Dense act-order: A's columns are gathered once into a_tmp by permute_cols (as the reference's
   // permute_cols_kernel, csrc/quantization/gptq_marlin/gptq_marlin.cu:68-120), so the GEMM kernels read A with
-  // plain 128-bit loads.  MoE blocks gather inside the kernel (rows and per-expert column order together).
-  pl.atmp_bytes = (act_order && !moe) ? a->size_m * a->size_k * 2 : 0;
-  const bool perm_in_kernel = act_order && moe;
+  // plain 128-bit loads.  MoE: rows and per-expert column order are gathered together, one row of a_tmp per sorted
+  // slot (moe_gather_rows), and the kernels read row `slot` instead of row id / top_k.
+  pl.atmp_bytes = act_order ? (moe ? a->n_sorted : a->size_m) * a->size_k * 2 : 0;
   // Prefill kernel: dense, at least one full 128-row tile's worth of rows, K a multiple of 128.
   const int64_t fat_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 512);
   // ... unless the same problem cut into 64-row tiles finishes sooner.  In units of one 128 x 512 tile's time (measured):
@@ -260,7 +260,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     int kps = (int)ceil_div(pl.total_ksteps, sp);
     kps = (kps + 3) / 4 * 4;
     sp = (int)ceil_div(pl.total_ksteps, kps);
-    const bool mid_shape = mid_ok && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX && !perm_in_kernel &&
+    const bool mid_shape = mid_ok && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX &&
                            (moe ? a->moe_block_size == 64
                                 : (a->size_m > 32 && (mid_tiles >= cus / 2 || (forced_kind == 3 && mid_tiles >= cus / 16))));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
@@ -385,7 +385,12 @@ static int run_planned(const w4a16_gemm_args* args, Plan& pl, void* stream) {
   w4a16_gemm_args b = *args;
   if (pl.atmp_bytes > 0) {
     void* a_tmp = (char*)args->c_tmp + ((pl.ctmp_bytes + 255) & ~255LL);
-    if (int rc = w4a16_permute_cols(args->a, args->perm, a_tmp, args->size_m, args->size_k, args->lda, stream)) return rc;
+    if (args->flags & W4A16_F_MOE) {
+      if (int rc = moe_gather_rows(args, a_tmp, (hipStream_t)stream)) return rc;
+      pl.a_by_slot = true;
+    } else {
+      if (int rc = w4a16_permute_cols(args->a, args->perm, a_tmp, args->size_m, args->size_k, args->lda, stream)) return rc;
+    }
     b.a = a_tmp;
     b.lda = args->size_k;
     pl.use_perm = false;

@@ -31,7 +31,7 @@ struct DecodeCfg {
   static constexpr int SMEM = DNW * 16 * RS * 4;
 };
 
-template <int DT, bool ZP, bool CHANNEL, bool PERM, int TN>
+template <int DT, bool ZP, bool CHANNEL, int TN>
 __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   constexpr int W = TN / 32;  // Marlin words per lane and k-tile: 4 (128-bit load) or 2 (64-bit load)
   constexpr bool HI_TRICK = (DT == DT_F16) && !ZP;
@@ -64,7 +64,6 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint32_t* Zp = p.Z;
-  const int32_t* perm = p.perm;
   const uint16_t* bias = (const uint16_t*)p.bias;
   if (p.moe) {
     if (mt * p.moe_bs >= *p.ntpp) return;
@@ -73,7 +72,6 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
     Bq += e * p.b_estride;
     Sc += e * p.s_estride;
     if (ZP) Zp += e * p.z_estride;
-    if (PERM) perm += e * p.k_estride;
     if (bias) bias += e * p.n_estride;
   }
 
@@ -84,7 +82,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
       if (r < p.moe_bs) {
         const int id = p.sorted_ids[mt * p.moe_bs + r];
         if ((unsigned)id < (unsigned)p.c_rows) {
-          src = id / p.top_k;
+          src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
           dst = id;
         }
       }
@@ -160,14 +158,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   auto issue = [&](Stage& s, int sidx) {  // sidx: absolute stage index (2 k-steps = 4 k-tiles = 64 K rows)
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      if constexpr (PERM) {
-        uint16_t e[8];
-        const uint16_t* row = arow[i] - ap * 8;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = row[perm[sidx * 64 + ap * 8 + j]];
-        s.a[i] = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
-                       (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
-      } else if (i == 1 && !rows_hi) {
+      if (i == 1 && !rows_hi) {
         s.a[i] = u32x4{0, 0, 0, 0};  // the tile has no rows 8..15
       } else {
         s.a[i] = *(const u32x4*)(arow[i] + sidx * 64);
@@ -456,24 +447,25 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
 // ------------------------------------------------------------------------------------ host side
 typedef void (*decode_fn)(const KParams);
 
-template <int DT, bool PERM, int TN>
+template <int DT, int TN>
 static decode_fn pick3(bool zp, bool channel) {
-  if (zp) return channel ? decode_kernel<DT, true, true, PERM, TN> : decode_kernel<DT, true, false, PERM, TN>;
-  return channel ? decode_kernel<DT, false, true, PERM, TN> : decode_kernel<DT, false, false, PERM, TN>;
+  if (zp) return channel ? decode_kernel<DT, true, true, TN> : decode_kernel<DT, true, false, TN>;
+  return channel ? decode_kernel<DT, false, true, TN> : decode_kernel<DT, false, false, TN>;
 }
-template <int DT, bool PERM>
+template <int DT>
 static decode_fn pick2(int tn, bool zp, bool channel) {
-  return tn == 64 ? pick3<DT, PERM, 64>(zp, channel) : pick3<DT, PERM, 128>(zp, channel);
+  return tn == 64 ? pick3<DT, 64>(zp, channel) : pick3<DT, 128>(zp, channel);
 }
 
-static decode_fn pick_decode(int dt, bool perm, int tn, bool zp, bool channel) {
-  if (dt == DT_F16) return perm ? pick2<DT_F16, true>(tn, zp, channel) : pick2<DT_F16, false>(tn, zp, channel);
-  return perm ? pick2<DT_BF16, true>(tn, zp, channel) : pick2<DT_BF16, false>(tn, zp, channel);
+// (act-order never reaches the kernel as such: the host gathers A's columns in front of the launch, see gemm.hip)
+static decode_fn pick_decode(int dt, int tn, bool zp, bool channel) {
+  return dt == DT_F16 ? pick2<DT_F16>(tn, zp, channel) : pick2<DT_BF16>(tn, zp, channel);
 }
 
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
-  decode_fn fn = pick_decode(a->dtype, pl.use_perm, pl.tn, zp, pl.gm == GM_CHANNEL);
+  if (pl.use_perm) return fail(W4A16_EINVAL, "unsupported kernel variant");
+  decode_fn fn = pick_decode(a->dtype, pl.tn, zp, pl.gm == GM_CHANNEL);
   KParams p = make_kparams(a, pl);
   const int smem = pl.tn == 64 ? DecodeCfg<64>::SMEM : DecodeCfg<128>::SMEM;
   W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));

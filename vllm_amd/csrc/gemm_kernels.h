@@ -14,7 +14,6 @@ struct KParams {
   const void* S;
   const uint32_t* Z;
   const int32_t* gidx;
-  const int32_t* perm;
   const void* bias;
   const void* gscale;  // NVFP4 global scale (one element of the activation type per expert), else null
   int fp8;             // weights are float8_e4m3fn (their stored scales carry an exponent offset)
@@ -40,6 +39,7 @@ struct KParams {
   int n_sorted;  // usable length of sorted_ids
   int64_t b_estride, s_estride, z_estride, k_estride, n_estride;  // per-expert strides (elements)
   // fused epilogues
+  int a_by_slot;  // MoE: row r of block mt reads A row mt * block + r (gathered in front of the launch), not id / top_k
   int act;        // 1: column halves are gate | up; C is [rows, N / 2] = silu(gate) * up
   int sum_div;    // > 0: result row i is added atomically into C row i / sum_div
   uint32_t* zero_ptr;  // side job: zero_n16 16-byte pieces to clear, spread over the grid
@@ -167,7 +167,6 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.S = a->b_scales;
   p.Z = a->b_zeros;
   p.gidx = pl.gm == GM_GIDX ? a->g_idx : nullptr;
-  p.perm = pl.use_perm ? a->perm : nullptr;
   p.bias = a->b_bias;
   p.gscale = a->global_scale;
   p.fp8 = a->wtype == W4A16_WTYPE_FE4M3;
@@ -205,6 +204,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.z_estride = a->num_groups * (a->size_n / 8);
   p.k_estride = a->size_k;
   p.n_estride = a->size_n;
+  p.a_by_slot = moe && pl.a_by_slot;
   p.act = moe && (a->flags & W4A16_F_SILU_AND_MUL);
   p.sum_div = (moe && (a->flags & W4A16_F_SUM_TOPK)) ? a->sum_top_k : 0;
   p.zero_ptr = (uint32_t*)a->zero_fill;

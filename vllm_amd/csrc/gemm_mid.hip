@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     if (MOE) {
       const int id = p.sorted_ids[row0 + r];
       if ((unsigned)id < (unsigned)p.c_rows) {
-        src = id / p.top_k;
+        src = p.a_by_slot ? row0 + r : id / p.top_k;
         dst = id;
       }
     } else if (row0 + r < p.M) {

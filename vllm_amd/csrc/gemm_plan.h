@@ -8,6 +8,7 @@ struct Plan {
   int gm;            // GM_*: how scale rows are found
   int group_ksteps;  // GM_GROUPED: group_size / 32
   bool use_perm;     // gather A columns through perm (act-order)
+  bool a_by_slot = false;  // MoE: A already holds one row per sorted slot (act-order gather done in front of the GEMM)
   int mb, bm;        // m-blocks of 16 rows per tile, rows per tile
   int mtiles, ncp, tiles;
   int total_ksteps, splits, kps;  // k-steps of 32 rows; K splits; k-steps per split
@@ -18,8 +19,12 @@ struct Plan {
   int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
   int tail_strips = 0; // prefill plan: trailing 512-column strips handed to the 64-row kernel (0 = none)
   int64_t ctmp_bytes;  // fp32 split-K partials
-  int64_t atmp_bytes;  // column-permuted copy of A (act-order in front of the prefill kernel), after the partials
+  int64_t atmp_bytes;  // column-permuted copy of A (act-order), after the partials; MoE: one row per sorted slot
 };
+
+// MoE act-order: out[slot, :] = a[sorted_ids[slot] / top_k, perm[expert of the slot's block][:]] for the valid slots
+// (gemm.hip runs it in front of the GEMM kernels, which then read row `slot`).
+int moe_gather_rows(const w4a16_gemm_args* a, void* out, hipStream_t stream);
 
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);

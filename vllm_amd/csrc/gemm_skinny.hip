@@ -39,13 +39,13 @@ struct SkinnyCfg {
 
 
 // FP4: 0 = integer weights, 1 = float4_e2m1f with NVFP4 scales (per k-tile), 2 = with MXFP4 scales (per k-step)
-template <int DT, int MB, bool ZP, int GM, bool PERM, int BITS = 4, bool ZPF = false, bool FP8 = false, int FP4 = 0>
+template <int DT, int MB, bool ZP, int GM, int BITS = 4, bool ZPF = false, bool FP8 = false, int FP4 = 0>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
   // ZPF: fp16 zero points laid out like the scales (HQQ); element-wise dequantisation on every tile size
-  static_assert(FP4 == 0 || (BITS == 4 && !ZP && !ZPF && GM == GM_GROUPED && !PERM), "fp4 weights: grouped scale records");
-  static_assert(!FP8 || (BITS == 8 && GM != GM_GIDX && !PERM), "fp8 weights use the 8-bit layout, no act-order");
-  static_assert(!ZPF || (DT == DT_F16 && !ZP && GM == GM_GROUPED && !PERM && BITS == 4), "float zero points: fp16 uint4 grouped");
+  static_assert(FP4 == 0 || (BITS == 4 && !ZP && !ZPF && GM == GM_GROUPED), "fp4 weights: grouped scale records");
+  static_assert(!FP8 || (BITS == 8 && GM != GM_GIDX), "fp8 weights use the 8-bit layout, no act-order");
+  static_assert(!ZPF || (DT == DT_F16 && !ZP && GM == GM_GROUPED && BITS == 4), "float zero points: fp16 uint4 grouped");
   constexpr int BM = 16 * MB;
   // 8-bit stages hold twice the weight registers: shorter ring
   // ... and so do the variants that keep extra per-stage state (per-row scale lookup, fp4 scale records)
@@ -90,7 +90,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint32_t* Zp = p.Z;
   const int32_t* gidx = p.gidx;
-  const int32_t* perm = p.perm;
   const uint16_t* bias = (const uint16_t*)p.bias;
   const uint16_t* gscale = (const uint16_t*)p.gscale;
   if (p.moe) {
@@ -102,7 +101,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     if (FP4 == 1) gscale += e;
     if (ZP) Zp += e * p.z_estride;
     if (gidx) gidx += e * p.k_estride;
-    if (PERM) perm += e * p.k_estride;
     if (bias) bias += e * p.n_estride;
   }
 
@@ -116,7 +114,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
       if (r < p.moe_bs) {
         const int id = p.sorted_ids[mt * p.moe_bs + r];
         if ((unsigned)id < (unsigned)p.c_rows) {
-          src = id / p.top_k;
+          src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
           dst = id;
         }
       }
@@ -184,16 +182,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   auto issue = [&](Stage& s, int ks) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      if constexpr (PERM) {
-        uint16_t e[8];
-        const uint16_t* row = arow[mb] - ap * 8;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = row[perm[ks * 32 + ap * 8 + j]];
-        s.a[mb] = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
-                        (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
-      } else {
-        s.a[mb] = *(const u32x4*)(arow[mb] + ks * 32);
-      }
+      s.a[mb] = *(const u32x4*)(arow[mb] + ks * 32);
     }
     int gi = 0;
     s.uni = true;
@@ -584,58 +573,46 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 // ------------------------------------------------------------------------------------ host side
 typedef void (*skinny_fn)(const KParams);
 
-template <int DT, int MB, bool PERM>
+template <int DT, int MB>
 static skinny_fn pick_zp_gm(bool zp, int gm) {
   if (zp) {
-    if (gm == GM_GROUPED) return skinny_kernel<DT, MB, true, GM_GROUPED, PERM>;
-    if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, true, GM_CHANNEL, PERM>;
+    if (gm == GM_GROUPED) return skinny_kernel<DT, MB, true, GM_GROUPED>;
+    if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, true, GM_CHANNEL>;
     return nullptr;
   }
-  if (gm == GM_GROUPED) return skinny_kernel<DT, MB, false, GM_GROUPED, PERM>;
-  if (gm == GM_CHANNEL) {
-    if constexpr (PERM) return nullptr; else return skinny_kernel<DT, MB, false, GM_CHANNEL, false>;
-  }
-  return skinny_kernel<DT, MB, false, GM_GIDX, PERM>;
+  if (gm == GM_GROUPED) return skinny_kernel<DT, MB, false, GM_GROUPED>;
+  if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, false, GM_CHANNEL>;
+  return skinny_kernel<DT, MB, false, GM_GIDX>;
 }
 
-template <int DT, bool PERM>
+template <int DT>
 static skinny_fn pick_mb(int mb, bool zp, int gm) {
   switch (mb) {
-    case 1: return pick_zp_gm<DT, 1, PERM>(zp, gm);
-    case 2: return pick_zp_gm<DT, 2, PERM>(zp, gm);
-    default: return pick_zp_gm<DT, 4, PERM>(zp, gm);
+    case 1: return pick_zp_gm<DT, 1>(zp, gm);
+    case 2: return pick_zp_gm<DT, 2>(zp, gm);
+    default: return pick_zp_gm<DT, 4>(zp, gm);
   }
 }
 
-template <int DT, bool PERM>
-static skinny_fn pick_w8(int mb, int gm) {  // uint8b128: no zero points; PERM: MoE act-order, A gathered in the kernel
-  if constexpr (PERM) {
-    if (gm == GM_CHANNEL) return nullptr;  // act-order needs groups
-  }
-  switch (mb) {
-    case 1:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, PERM, 8>
-             : gm == GM_CHANNEL ? skinny_kernel<DT, 1, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 1, false, GM_GIDX, PERM, 8>;
-    case 2:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, PERM, 8>
-             : gm == GM_CHANNEL ? skinny_kernel<DT, 2, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 2, false, GM_GIDX, PERM, 8>;
-    default:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, PERM, 8>
-             : gm == GM_CHANNEL ? skinny_kernel<DT, 4, false, GM_CHANNEL, false, 8>
-                                : skinny_kernel<DT, 4, false, GM_GIDX, PERM, 8>;
-  }
+template <int DT, int MB>
+static skinny_fn pick_w8_gm(int gm) {  // uint8b128: no zero points
+  return gm == GM_GROUPED ? skinny_kernel<DT, MB, false, GM_GROUPED, 8>
+         : gm == GM_CHANNEL ? skinny_kernel<DT, MB, false, GM_CHANNEL, 8>
+                            : skinny_kernel<DT, MB, false, GM_GIDX, 8>;
 }
 
-static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool perm, bool w8) {
+template <int DT>
+static skinny_fn pick_w8(int mb, int gm) {
+  return mb == 1 ? pick_w8_gm<DT, 1>(gm) : mb == 2 ? pick_w8_gm<DT, 2>(gm) : pick_w8_gm<DT, 4>(gm);
+}
+
+// (act-order never reaches a kernel as such: the host gathers A's columns in front of the launch, see gemm.hip)
+static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool w8) {
   if (w8) {
     if (zp) return nullptr;
-    if (perm) return dt == DT_F16 ? pick_w8<DT_F16, true>(mb, gm) : pick_w8<DT_BF16, true>(mb, gm);
-    return dt == DT_F16 ? pick_w8<DT_F16, false>(mb, gm) : pick_w8<DT_BF16, false>(mb, gm);
+    return dt == DT_F16 ? pick_w8<DT_F16>(mb, gm) : pick_w8<DT_BF16>(mb, gm);
   }
-  if (perm) return dt == DT_F16 ? pick_mb<DT_F16, true>(mb, zp, gm) : pick_mb<DT_BF16, true>(mb, zp, gm);
-  return dt == DT_F16 ? pick_mb<DT_F16, false>(mb, zp, gm) : pick_mb<DT_BF16, false>(mb, zp, gm);
+  return dt == DT_F16 ? pick_mb<DT_F16>(mb, zp, gm) : pick_mb<DT_BF16>(mb, zp, gm);
 }
 
 static int skinny_smem_bytes(int mb) {
@@ -646,31 +623,31 @@ template <int DT>
 static skinny_fn pick_fp8(int mb, int gm) {  // float8_e4m3fn: grouped or channel-wise scales, no act-order
   switch (mb) {
     case 1:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, false, 8, false, true>
-                              : skinny_kernel<DT, 1, false, GM_CHANNEL, false, 8, false, true>;
+      return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, 8, false, true>
+                              : skinny_kernel<DT, 1, false, GM_CHANNEL, 8, false, true>;
     case 2:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, false, 8, false, true>
-                              : skinny_kernel<DT, 2, false, GM_CHANNEL, false, 8, false, true>;
+      return gm == GM_GROUPED ? skinny_kernel<DT, 2, false, GM_GROUPED, 8, false, true>
+                              : skinny_kernel<DT, 2, false, GM_CHANNEL, 8, false, true>;
     default:
-      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, false, 8, false, true>
-                              : skinny_kernel<DT, 4, false, GM_CHANNEL, false, 8, false, true>;
+      return gm == GM_GROUPED ? skinny_kernel<DT, 4, false, GM_GROUPED, 8, false, true>
+                              : skinny_kernel<DT, 4, false, GM_CHANNEL, 8, false, true>;
   }
 }
 
 template <int DT, int FP4>
 static skinny_fn pick_fp4(int mb) {  // float4_e2m1f (validated on the host: grouped records, no act-order, dense)
   switch (mb) {
-    case 1: return skinny_kernel<DT, 1, false, GM_GROUPED, false, 4, false, false, FP4>;
-    case 2: return skinny_kernel<DT, 2, false, GM_GROUPED, false, 4, false, false, FP4>;
-    default: return skinny_kernel<DT, 4, false, GM_GROUPED, false, 4, false, false, FP4>;
+    case 1: return skinny_kernel<DT, 1, false, GM_GROUPED, 4, false, false, FP4>;
+    case 2: return skinny_kernel<DT, 2, false, GM_GROUPED, 4, false, false, FP4>;
+    default: return skinny_kernel<DT, 4, false, GM_GROUPED, 4, false, false, FP4>;
   }
 }
 
 static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
   switch (mb) {
-    case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, false, 4, true>;
-    case 2: return skinny_kernel<DT_F16, 2, false, GM_GROUPED, false, 4, true>;
-    default: return skinny_kernel<DT_F16, 4, false, GM_GROUPED, false, 4, true>;
+    case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, 4, true>;
+    case 2: return skinny_kernel<DT_F16, 2, false, GM_GROUPED, 4, true>;
+    default: return skinny_kernel<DT_F16, 4, false, GM_GROUPED, 4, true>;
   }
 }
 
@@ -683,12 +660,12 @@ int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
     fn = a->global_scale ? (a->dtype == DT_F16 ? pick_fp4<DT_F16, 1>(pl.mb) : pick_fp4<DT_BF16, 1>(pl.mb))
                          : pick_fp4<DT_BF16, 2>(pl.mb);
   else if (a->wtype == W4A16_WTYPE_FE4M3)
-    fn = (pl.gm == GM_GIDX || pl.use_perm) ? nullptr
-         : a->dtype == DT_F16              ? pick_fp8<DT_F16>(pl.mb, pl.gm)
-                                           : pick_fp8<DT_BF16>(pl.mb, pl.gm);
+    fn = pl.gm == GM_GIDX     ? nullptr
+         : a->dtype == DT_F16 ? pick_fp8<DT_F16>(pl.mb, pl.gm)
+                              : pick_fp8<DT_BF16>(pl.mb, pl.gm);
   else
-    fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, pl.use_perm, a->wtype == W4A16_WTYPE_U8B128);
-  if (!fn) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, a->wtype == W4A16_WTYPE_U8B128);
+  if (!fn || pl.use_perm) return fail(W4A16_EINVAL, "unsupported kernel variant");
   KParams p = make_kparams(a, pl);
   const int smem = skinny_smem_bytes(pl.mb);
   W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));

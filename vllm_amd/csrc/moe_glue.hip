@@ -300,6 +300,74 @@ extern "C" int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel
   return 0;
 }
 
+// MoE act-order gather in front of the GEMM (the role of the reference's permute_cols_kernel<moe_block_size>,
+// csrc/moe/marlin_moe_wna16/ops.cu:75-149): out[slot, k] = a[sorted_ids[slot] / top_k, perm_e[k]] for every valid slot,
+// perm_e = the column order of the expert that owns the slot's block.  One workgroup per slot and turn: the source row is
+// staged in LDS with 16-byte loads, every thread assembles 16-byte pieces of the output row from eight 2-byte LDS reads.
+// Slots past the padded total, padding slots and blocks of experts of other ranks are skipped (their rows of `out` stay
+// as they are: the GEMM kernels never store results of such rows).
+namespace w4a16 {
+constexpr int MG_MAX_K = 32768;  // 64 KB of LDS
+template <bool STAGED>
+__global__ __launch_bounds__(256) void moe_gather_rows_kernel(const uint16_t* __restrict__ a, int64_t lda,
+                                                             const int32_t* __restrict__ perm,
+                                                             const int32_t* __restrict__ sorted_ids,
+                                                             const int32_t* __restrict__ expert_ids,
+                                                             const int32_t* __restrict__ ntpp, int n_sorted, int block,
+                                                             int top_k, int c_rows, int size_k,
+                                                             uint16_t* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char mg_smem[];
+  uint16_t* row = (uint16_t*)mg_smem;
+  const int t = threadIdx.x;
+  const int total = min(*ntpp, n_sorted);
+  const int pieces = size_k >> 3;
+  for (int slot = blockIdx.x; slot < total; slot += gridDim.x) {
+    const int id = sorted_ids[slot];
+    const int e = expert_ids[slot / block];
+    if ((unsigned)id >= (unsigned)c_rows || e < 0) continue;  // (uniform over the workgroup)
+    const uint16_t* src = a + (int64_t)(id / top_k) * lda;
+    const int32_t* pe = perm + (int64_t)e * size_k;
+    uint16_t* dst = out + (int64_t)slot * size_k;
+    if constexpr (STAGED) {
+      __syncthreads();  // the previous turn's gathers are done
+      for (int p = t; p < pieces; p += 256) ((u32x4*)row)[p] = ((const u32x4*)src)[p];
+      __syncthreads();
+      for (int p = t; p < pieces; p += 256) {
+        const u32x4 i0 = *(const u32x4*)(pe + 8 * p), i1 = *(const u32x4*)(pe + 8 * p + 4);
+        u32x4 v;
+        v[0] = (uint32_t)row[i0[0]] | ((uint32_t)row[i0[1]] << 16);
+        v[1] = (uint32_t)row[i0[2]] | ((uint32_t)row[i0[3]] << 16);
+        v[2] = (uint32_t)row[i1[0]] | ((uint32_t)row[i1[1]] << 16);
+        v[3] = (uint32_t)row[i1[2]] | ((uint32_t)row[i1[3]] << 16);
+        ((u32x4*)dst)[p] = v;
+      }
+    } else {
+      for (int k = t; k < size_k; k += 256) dst[k] = src[pe[k]];
+    }
+  }
+}
+
+int moe_gather_rows(const w4a16_gemm_args* a, void* out, hipStream_t stream) {
+  const int64_t k = a->size_k;
+  if (a->n_sorted <= 0 || k == 0) return 0;
+  const int64_t slots = a->n_sorted;
+  const unsigned grid = (unsigned)(slots < 8 * (int64_t)num_cus() ? slots : 8 * (int64_t)num_cus());
+  const int c_rows = (int)(a->size_m * a->top_k);
+  const bool staged = k % 8 == 0 && k <= MG_MAX_K && a->lda % 8 == 0 && ((uintptr_t)a->a & 15) == 0 &&
+                      ((uintptr_t)out & 15) == 0 && ((uintptr_t)a->perm & 15) == 0;
+  if (staged)
+    moe_gather_rows_kernel<true><<<grid, 256, (size_t)k * 2, stream>>>(
+        (const uint16_t*)a->a, a->lda, a->perm, a->sorted_token_ids, a->expert_ids, a->num_tokens_past_padded,
+        (int)a->n_sorted, a->moe_block_size, a->top_k, c_rows, (int)k, (uint16_t*)out);
+  else
+    moe_gather_rows_kernel<false><<<grid, 256, 0, stream>>>(
+        (const uint16_t*)a->a, a->lda, a->perm, a->sorted_token_ids, a->expert_ids, a->num_tokens_past_padded,
+        (int)a->n_sorted, a->moe_block_size, a->top_k, c_rows, (int)k, (uint16_t*)out);
+  W4A16_HIP(hipGetLastError());
+  return 0;
+}
+}  // namespace w4a16
+
 extern "C" int w4a16_moe_sum(const void* in, void* out, int64_t tokens, int32_t top_k, int64_t hidden,
                              int32_t dtype, void* stream) {
   W4A16_CHECK(in && out, "null pointer");
