@@ -33,7 +33,8 @@ constexpr int NW = 8;        // wavefronts per workgroup
 
 template <int MB>
 struct SkinnyCfg {
-  static constexpr int D = (MB >= 4) ? 3 : 6;  // k-steps in flight per wavefront
+  // k-steps in flight per wavefront (measured: deeper rings on the taller tiles cost registers, hence spills, and time)
+  static constexpr int D = (MB >= 4) ? 2 : (MB == 2) ? 4 : 6;
   static constexpr int SMEM = NW * 16 * RED_RS * 4;  // reduction slab; its head doubles as the A bounce slabs
 };
 
@@ -49,9 +50,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   constexpr int BM = 16 * MB;
   // 8-bit stages hold twice the weight registers: shorter ring
   // ... and so do the variants that keep extra per-stage state (per-row scale lookup, fp4 scale records)
-  // ... and the 64-row channel-wise variants, which otherwise spill inside the loop
-  constexpr int D = (BITS == 8) ? (MB >= 4 ? 2 : 3)
-                    : ((FP4 != 0 || GM == GM_GIDX) && MB >= 2) || (GM == GM_CHANNEL && MB >= 4) ? 2 : SkinnyCfg<MB>::D;
+  constexpr int D = (BITS == 8) ? (MB >= 4 ? 2 : 3) : ((FP4 != 0 || GM == GM_GIDX) && MB >= 2) ? 2 : SkinnyCfg<MB>::D;
   constexpr bool UNIT = (GM == GM_CHANNEL);
   // Decode tiles (one m-block) keep the weights as raw magic numbers E+q in the MFMA and apply
   // "-(E+z)" and the group scale to the fp32 accumulator once per group (see fold() below).
