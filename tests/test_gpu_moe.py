@@ -255,6 +255,28 @@ def test_fused_marlin_moe_vs_torch_moe(dev, m, e, topk, variant):
     torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
 
 
+@pytest.mark.parametrize("m", [1, 16, 300])
+@pytest.mark.parametrize("e,topk", [(64, 6), (128, 8)])
+def test_fused_marlin_moe_many_experts(dev, m, e, topk):
+    """Expert counts and top-k of the fine-grained MoE models (64 experts / top-6, 128 / top-8): most blocks hold one or
+    two slots, top-k above 2 takes the five-launch sequence.  Same gate as above."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    dtype, k, inter = torch.float16, 256, 128
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=500)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 128, dtype, False, False, seed=700)
+    g = torch.Generator().manual_seed(13)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    score = torch.randn(m, e, generator=g).to(dtype)
+    tw, ti = torch.topk(torch.softmax(score.float(), dim=-1), topk)
+    tw = tw / tw.sum(dim=-1, keepdim=True)
+    out = fused_marlin_moe(a.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), score.to(dev),
+                           tw.to(dev), ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e)
+    w1 = torch.stack([l.w_ref.t() for l in l1])
+    w2 = torch.stack([l.w_ref.t() for l in l2])
+    ref = mr.torch_experts(a, w1, w2, tw, ti)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
+
+
 def test_fused_marlin_moe_mixtral_shape(dev):
     """Mixtral-8x7B expert shapes (hidden 4096, intermediate 14336, top-2) at T = 16; two experts instead of
     eight, so that quantising them with the CPU oracle stays within seconds."""

@@ -95,31 +95,39 @@ def _run_experts(x: torch.Tensor, ex: _Experts, rt: _Routing, weight_on_input: b
     slots = m * rt.topk
     dev, dt = x.device, x.dtype
     act = inter_buf.view(-1)[:slots * n].view(slots, n) if inter_buf is not None else torch.empty((slots, n), device=dev, dtype=dt)
-    fusable = activation == "silu" and activation_func is default_activation_func and moe_sum is None
-    if fusable and (rt.topk <= 2 or not reduce_topk):
-        if out is None:
-            out = torch.empty((m if reduce_topk else slots, k), device=dev, dtype=dt)
-        summing = reduce_topk and rt.topk == 2
-        needs_zero = summing or rt.expert_parallel       # rows of experts on other ranks are never written
-        aliased = out is x                                # inplace: GEMM1 still reads what the side job would clear
-        side_job = out if needs_zero and not aliased and out.is_contiguous() else None
+    # what the GEMM launches can take over: SiLU-and-mul in GEMM1's epilogue whenever the default activation is asked
+    # for; the top-k sum in GEMM2's epilogue for two terms (a sum of two does not depend on their order)
+    act_fused = activation == "silu" and activation_func is default_activation_func
+    sum_fused = reduce_topk and moe_sum is None and rt.topk == 2
+    direct = not reduce_topk or (moe_sum is None and rt.topk == 1)   # GEMM2 writes the result rows themselves
+    if (sum_fused or direct) and out is None:
+        out = torch.empty((m if reduce_topk else slots, k), device=dev, dtype=dt)
+    needs_zero = sum_fused or (direct and rt.expert_parallel)    # rows of experts on other ranks are never written
+    big = max(0 if act_fused else 2 * n, 0 if (sum_fused or direct) else k)
+    shared = None
+    if big:
+        shared = gemm_buf if gemm_buf is not None else torch.empty((slots * big,), device=dev, dtype=dt)
+    # ---- GEMM1 (+ activation)
+    cleared = False
+    if act_fused:
+        # the launch can clear GEMM2's output on the side, unless GEMM1 still reads it (inplace) or it is a strided view
+        side_job = out if needs_zero and out is not x and out.is_contiguous() else None
         _gemm(ex, 0, rt, x, act, m, 2 * n, k, rt.topk, weight_on_input, silu_and_mul=True, sum_top_k=0, zero_fill=side_job)
-        if needs_zero and side_job is None:
+        cleared = side_job is not None
+    else:
+        h = _gemm(ex, 0, rt, x, shared.view(-1)[:slots * 2 * n].view(slots, 2 * n), m, 2 * n, k, rt.topk, weight_on_input)
+        activation_func(activation, act, h)
+    # ---- GEMM2 (+ top-k sum)
+    if sum_fused or direct:
+        if needs_zero and not cleared:
             out.zero_()
         _gemm(ex, 1, rt, act, out, slots, k, n, 1, not weight_on_input, silu_and_mul=False,
-              sum_top_k=2 if summing else 0, zero_fill=None)
+              sum_top_k=2 if sum_fused else 0, zero_fill=None)
         return out
-    # general sequence: separate activation and top-k sum
-    big = max(2 * n, k)
-    shared = gemm_buf if gemm_buf is not None else torch.empty((slots * big,), device=dev, dtype=dt)
-    h = _gemm(ex, 0, rt, x, shared.view(-1)[:slots * 2 * n].view(slots, 2 * n), m, 2 * n, k, rt.topk, weight_on_input)
-    activation_func(activation, act, h)
-    y = shared.view(-1)[:slots * k].view(slots, k) if reduce_topk or out is None else out
+    y = shared.view(-1)[:slots * k].view(slots, k)
     if rt.expert_parallel:
         y.zero_()
     y = _gemm(ex, 1, rt, act, y, slots, k, n, 1, not weight_on_input)
-    if not reduce_topk:
-        return y
     if out is None:
         out = torch.empty((m, k), device=dev, dtype=dt)
     y3 = y.view(m, rt.topk, k)
