@@ -25,7 +25,11 @@ def test_align_docstring_example(dev):
 
 
 @pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 8, 8), (16, 2, 8, 16), (123, 3, 12, 32), (666, 2, 4, 64),
-                                         (4096, 2, 8, 64), (1000, 6, 256, 16), (3, 8, 1024, 8)])
+                                         (4096, 2, 8, 64), (1000, 6, 256, 16), (3, 8, 1024, 8),
+                                         # both kernels behind the op, one and several staged chunks of ids, an id
+                                         # count that is no multiple of anything, more experts than the ranked kernel takes
+                                         (512, 2, 8, 64), (9000, 2, 8, 64), (4321, 8, 200, 48), (2500, 7, 256, 64),
+                                         (700, 3, 300, 16), (20000, 1, 3, 64)])
 @pytest.mark.parametrize("pad", [False, True])
 def test_align_equals_oracle(dev, m, topk, e, bs, pad):
     from vllm_amd.moe_align_block_size import moe_align_block_size
