@@ -248,8 +248,13 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     const int64_t mid_mtiles = moe ? ceil_div(a->n_sorted, 64) : ceil_div(a->size_m, 64);
     const int64_t mid_tiles = mid_mtiles * ceil_div(a->size_n, 512);
     int sp = 1;
+    // 8-bit weights at 65..128 rows: the general kernel would stream the (twice as large) weights once per 64-row tile;
+    // two K splits of the 64-row kernel win from cus/4 tiles on (gate_up, 96 / 128 rows: 81 / 85 -> 66 / 67 us)
+    const bool w8_two_tiles = w8 && !moe && a->size_m > 64 && a->size_m <= 128 && mid_tiles >= cus / 4 && mid_tiles < cus / 2;
     // (measured: worth it from about cus/2 tiles up to 3/4 cus dense, up to cus for MoE, whose tile count is an upper bound)
-    if ((mid_tiles >= cus / 2 || forced_kind == 3) && mid_tiles < (moe ? cus : cus * 3 / 4)) {
+    if (w8_two_tiles) {
+      sp = 2;
+    } else if ((mid_tiles >= cus / 2 || forced_kind == 3) && mid_tiles < (moe ? cus : cus * 3 / 4)) {
       const int by_k = pl.total_ksteps / 32;
       const int by_cus = (int)(2 * cus / mid_tiles);
       sp = by_k < by_cus ? by_k : by_cus;
@@ -262,7 +267,8 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     sp = (int)ceil_div(pl.total_ksteps, kps);
     const bool mid_shape = mid_ok && pow2_group && a->size_k % 128 == 0 && pl.gm != GM_GIDX &&
                            (moe ? a->moe_block_size == 64
-                                : (a->size_m > 32 && (mid_tiles >= cus / 2 || (forced_kind == 3 && mid_tiles >= cus / 16))));
+                                : (a->size_m > 32 && (mid_tiles >= cus / 2 || w8_two_tiles ||
+                                                      (forced_kind == 3 && mid_tiles >= cus / 16))));
     if ((mid_shape && forced_kind < 0) || (forced_kind == 3 && mid_shape)) {
       W4A16_CHECK(mid_tiles * sp < (1LL << 31) / 64, "too many tiles");
       pl.kind = 3;
