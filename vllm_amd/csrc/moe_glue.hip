@@ -91,6 +91,156 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(
   }
 }
 
+// The same contract for long id lists (prefill): the kernel above walks all ids once per expert with one wavefront, four
+// dependent 4-byte loads per round trip, and re-reads them with as many round trips for the histogram; here
+//   * every thread fetches its ids with 16-byte loads, several in flight, for the histogram (LDS atomics: per-expert
+//     ballot counts for the few-expert case, where lanes queue on a few addresses, measured slower);
+//   * the ids of an expert are placed by `spe` wavefronts of a workgroup, each on a contiguous slice of the ids:
+//     count the matches of the slice, exchange the counts through LDS, place from the slice's start position.  A lane
+//     holds four consecutive ids; a match's rank is the matches of the lanes in front plus its own earlier components,
+//     so the order inside an expert stays the order of the ids (stable, deterministic).
+using i32x4 = int32_t __attribute__((ext_vector_type(4)));
+constexpr int ALIGN_ROUND = 8;  // 16-byte loads in flight per lane in the placement passes (2048 ids per wavefront round)
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_sliced_kernel(
+    const int32_t* __restrict__ topk_ids, int numel, int num_experts, int block_size, int spe,
+    int32_t* __restrict__ sorted_ids, int sorted_len, int32_t* __restrict__ expert_ids, int expert_ids_len,
+    int32_t* __restrict__ num_post_pad) {
+  __shared__ int cnt[ALIGN_MAX_EXPERTS];
+  __shared__ int off[ALIGN_MAX_EXPERTS + 1];
+  __shared__ int slice_cnt[ALIGN_WAVES];
+  const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  for (int e = t; e < num_experts; e += ALIGN_THREADS) cnt[e] = 0;
+  __syncthreads();
+  const int nvec = numel >> 2;  // whole 16-byte groups; the last numel & 3 ids are handled one by one
+  const i32x4* vids = (const i32x4*)topk_ids;
+
+  // ---- histogram
+  for (int v0 = 0; v0 < nvec; v0 += 4 * ALIGN_THREADS) {
+    i32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int vi = v0 + j * ALIGN_THREADS + t;
+      v[j] = vi < nvec ? vids[vi] : i32x4{-1, -1, -1, -1};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int e = v[j][q];
+        if (e >= 0 && e < num_experts) atomicAdd(&cnt[e], 1);
+      }
+    }
+  }
+  if (t < (numel & 3)) {
+    const int e = topk_ids[4 * nvec + t];
+    if (e >= 0 && e < num_experts) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (t < 64) {  // wave 0: exclusive scan of padded counts, 64 experts per round
+    int acc = 0;
+    for (int base = 0; base < num_experts; base += 64) {
+      const int e = base + t;
+      const int padded = e < num_experts ? (cnt[e] + block_size - 1) / block_size * block_size : 0;
+      int incl = padded;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_up(incl, d, 64);
+        if (t >= d) incl += v;
+      }
+      if (e < num_experts) off[e] = acc + incl - padded;
+      acc += __shfl(incl, 63, 64);
+    }
+    if (t == 0) off[num_experts] = acc;
+  }
+  __syncthreads();
+  const int total = off[num_experts];
+  if (blockIdx.x == 0) {
+    if (t == 0) *num_post_pad = total;
+    // expert id of every block; blocks past the padded total are zero-filled; slots past the total hold numel
+    for (int e = t; e < num_experts; e += ALIGN_THREADS) {
+      const int b0 = off[e] / block_size, b1 = off[e + 1] / block_size;
+      for (int b = b0; b < b1 && b < expert_ids_len; ++b) expert_ids[b] = e;
+    }
+    for (int b = total / block_size + t; b < expert_ids_len; b += ALIGN_THREADS) expert_ids[b] = 0;
+    for (int i = total + t; i < sorted_len; i += ALIGN_THREADS) sorted_ids[i] = numel;
+  }
+
+  // ---- placement: workgroup turn `eg` handles experts eg * epw .. + epw - 1, `spe` wavefronts each
+  const int epw = ALIGN_WAVES / spe;
+  const int j = wv / spe, sl = wv % spe;
+  // slice of the 16-byte groups: whole wavefront loads (64 groups)
+  const int per = ((nvec + spe - 1) / spe + 63) / 64 * 64;
+  const int vb = min(sl * per, nvec), ve = min(vb + per, nvec);
+  for (int eg = blockIdx.x; eg * epw < num_experts; eg += gridDim.x) {
+    const int e = eg * epw + j;
+    const bool live = e < num_experts && cnt[e] > 0;
+    // matches of expert e in groups [vb, ve): pass 0 counts, pass 1 places from `pos`
+    int pos = 0;
+    for (int pass = 0; pass < 2; ++pass) {
+      int seen = 0;
+      if (live) {
+        for (int v0 = vb; v0 < ve; v0 += 64 * ALIGN_ROUND) {
+          i32x4 v[ALIGN_ROUND];
+#pragma unroll
+          for (int r = 0; r < ALIGN_ROUND; ++r) {
+            const int vi = v0 + 64 * r + lane;
+            v[r] = vi < ve ? vids[vi] : i32x4{-1, -1, -1, -1};
+          }
+#pragma unroll
+          for (int r = 0; r < ALIGN_ROUND; ++r) {
+            unsigned long long m[4];
+            int before = 0, all = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              m[q] = __ballot(v[r][q] == e);
+              before += __popcll(m[q] & lt);
+              all += __popcll(m[q]);
+            }
+            if (pass == 1 && all) {
+              int p = pos + seen + before;
+              const int idx = 4 * (v0 + 64 * r + lane);
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if (v[r][q] == e) {
+                  if (p < sorted_len) sorted_ids[p] = idx + q;
+                  ++p;
+                }
+              }
+            }
+            seen += all;
+          }
+        }
+        // the last slice also owns the numel & 3 ids past the 16-byte groups
+        if (sl == spe - 1) {
+          const int i = 4 * nvec + lane;
+          const bool hit = lane < (numel & 3) && topk_ids[i] == e;
+          const unsigned long long m = __ballot(hit);
+          if (pass == 1 && hit) {
+            const int p = pos + seen + __popcll(m & lt);
+            if (p < sorted_len) sorted_ids[p] = i;
+          }
+          seen += __popcll(m);
+        }
+      }
+      if (pass == 0) {
+        if (lane == 0) slice_cnt[wv] = seen;
+        __syncthreads();
+        if (live) {
+          pos = off[e];
+          for (int s2 = 0; s2 < sl; ++s2) pos += slice_cnt[j * spe + s2];
+        }
+        __syncthreads();  // slice_cnt is rewritten in the next turn
+      }
+    }
+    // padding slots of the expert: by its first slice's wavefront
+    if (e < num_experts && sl == 0) {
+      const int padded = (cnt[e] + block_size - 1) / block_size * block_size;
+      for (int i = off[e] + cnt[e] + lane; i < off[e] + padded && i < sorted_len; i += 64) sorted_ids[i] = numel;
+    }
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
                                                       int64_t total8, int top_k, int64_t hidden8) {
@@ -292,6 +442,18 @@ extern "C" int w4a16_moe_align_block_size(const int32_t* topk_ids, int64_t numel
   W4A16_CHECK(block_size >= 1, "block_size must be positive");
   W4A16_CHECK(numel >= 0 && numel < (1LL << 30), "bad topk_ids.numel()");
   W4A16_CHECK(sorted_len >= numel, "sorted_token_ids is shorter than topk_ids");
+  if (numel >= 2048 && ((uintptr_t)topk_ids & 15) == 0) {
+    // slices per expert: enough wavefronts for 64 and more workgroups, slices of at least 256 ids
+    int spe = 1;
+    while (spe < ALIGN_WAVES && num_experts * spe < 1024 && numel / (2 * spe) >= 256) spe *= 2;
+    const int64_t turns = ceil_div(num_experts, ALIGN_WAVES / spe);
+    const int grid = (int)(turns < 256 ? turns : 256);
+    moe_align_sliced_kernel<<<grid, ALIGN_THREADS, 0, (hipStream_t)stream>>>(
+        topk_ids, (int)numel, num_experts, block_size, spe, sorted_token_ids, (int)sorted_len, expert_ids,
+        (int)expert_ids_len, num_tokens_post_pad);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
   const int grid = (int)ceil_div(num_experts, ALIGN_WAVES);
   moe_align_kernel<<<grid, ALIGN_THREADS, 0, (hipStream_t)stream>>>(
       topk_ids, (int)numel, num_experts, block_size, sorted_token_ids, (int)sorted_len, expert_ids,
