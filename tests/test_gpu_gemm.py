@@ -381,3 +381,23 @@ def test_one_row_tile_of_256_columns(ops, dev, workspace, dtype, mode, group):
     out = run_gemm(ops, layer, hot.to(dev), dev, workspace)
     assert torch.equal(out.cpu(), layer.w_ref[ks])
     assert int(workspace.abs().sum()) == 0
+
+
+# ------------------------------------------------- decode kernel with more column tiles than compute units
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("has_zp,group_size", [(False, 128), (True, 128), (False, -1), (True, 64)])
+def test_decode_more_tiles_than_compute_units(ops, dev, workspace, dtype, has_zp, group_size):
+    """N / 128 = 320 column tiles: the launch runs as 4-wavefront workgroups, two to a compute unit, whose final phase
+    walks the tile's 16 rows in two passes.  One-hot rows bit for bit, random rows within the GEMM tolerance."""
+    size_k, size_n = 256, 128 * 320
+    print(f"wide decode dtype={dtype} zp={has_zp} g={group_size}", flush=True)
+    layer = make_layer(size_k, size_n, group_size, dtype, has_zp=has_zp, seed=21)
+    ks = torch.tensor([0, 1, 9, 15, 16, 31, 32, 63, 64, 100, 127, 128, 200, 254, 255, 77])
+    a = torch.zeros(16, size_k, dtype=dtype)
+    a[torch.arange(16), ks] = 1.0
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    for m in (3, 13):  # rows 8..15 absent / present
+        a = _a(m, size_k, dtype, dev, seed=22 + m)
+        check_close(run_gemm(ops, layer, a, dev, workspace), a, layer)
+    assert int(workspace.abs().sum()) == 0

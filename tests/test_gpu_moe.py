@@ -281,6 +281,29 @@ def test_fused_marlin_moe_many_experts(dev, m, e, topk):
     torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,topk", [(64, 2), (24, 8)])
+def test_fused_marlin_moe_more_tiles_than_compute_units(dev, dtype, m, topk):
+    """128 experts, blocks of a few slots and four column tiles per block: both GEMMs launch more 16-row tiles than the
+    chip has compute units, which the decode kernel runs as 4-wavefront workgroups (fused SiLU-and-mul epilogue, and for
+    top-2 the fused sum, on that variant).  Same gate as above."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    e, k, inter = 128, 512, 256
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=900)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 128, dtype, False, False, seed=1100)
+    g = torch.Generator().manual_seed(14)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    score = torch.randn(m, e, generator=g).to(dtype)
+    tw, ti = torch.topk(torch.softmax(score.float(), dim=-1), topk)
+    tw = tw / tw.sum(dim=-1, keepdim=True)
+    out = fused_marlin_moe(a.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), score.to(dev),
+                           tw.to(dev), ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e)
+    w1 = torch.stack([l.w_ref.t() for l in l1])
+    w2 = torch.stack([l.w_ref.t() for l in l2])
+    ref = mr.torch_experts(a, w1, w2, tw, ti)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
+
+
 def test_fused_marlin_moe_mixtral_shape(dev):
     """Mixtral-8x7B expert shapes (hidden 4096, intermediate 14336, top-2) at T = 16; two experts instead of
     eight, so that quantising them with the CPU oracle stays within seconds."""

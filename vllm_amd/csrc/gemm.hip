@@ -160,8 +160,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   static const int forced_tn = env_int("W4A16_TN", 0);
   static const int forced_kind = env_int("W4A16_KIND", -1);
   static const int debug_plan = env_int("W4A16_DEBUG", 0);
+  static const int forced_nw = env_int("W4A16_NW", 0);
 #else
-  constexpr int forced_splits = 0, forced_tn = 0, forced_kind = -1, debug_plan = 0;
+  constexpr int forced_splits = 0, forced_tn = 0, forced_kind = -1, debug_plan = 0, forced_nw = 0;
 #endif
 
   // Dense act-order: A's columns are gathered once into a_tmp by permute_cols (as the reference's
@@ -365,10 +366,12 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = kps;
     pl.splits = (int)ceil_div(pl.total_ksteps, kps);
   }
+  // decode kernel: more workgroups than compute units -> 4-wavefront workgroups, two to a compute unit
+  pl.nw = forced_nw ? forced_nw : (pl.kind == 1 && (int64_t)pl.tiles * pl.splits > cus) ? 4 : 8;
   if (debug_plan)
-    fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=%d tn=%d mb=%d tiles=%d splits=%d kps=%d model_us=%.2f\n",
+    fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=%d tn=%d mb=%d tiles=%d splits=%d kps=%d nw=%d model_us=%.2f\n",
             (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, pl.kind, pl.tn, pl.mb, pl.tiles,
-            pl.splits, pl.kps, best.t);
+            pl.splits, pl.kps, pl.nw, best.t);
   pl.xcd_map = (pl.splits > 1 && pl.tiles % 8 == 0) ? 1 : 0;
   pl.ctmp_bytes = pl.splits > 1 ? (int64_t)pl.tiles * pl.splits * pl.bm * pl.tn * 4 : 0;
   return 0;

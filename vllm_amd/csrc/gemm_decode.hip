@@ -22,17 +22,19 @@
 
 namespace w4a16 {
 
-constexpr int DNW = 8;  // wavefronts per workgroup
+// Wavefronts per workgroup: 8, or 4 when a launch has several workgroups per compute unit in turn: two 4-wavefront
+// workgroups share a compute unit (same registers and loads in flight as one of 8), so one's prologue and
+// epilogue latencies run under the other's weight stream.
 constexpr int DD = 3;   // stages (of two k-steps) in flight per wavefront
 
 template <int TN>
 struct DecodeCfg {
   static constexpr int RS = (TN == 128) ? RED_RS : 84;  // reduction slab row stride (floats), 4 mod 16
-  static constexpr int SMEM = DNW * 16 * RS * 4;
+  static constexpr int smem(int nw) { return nw * 16 * RS * 4; }
 };
 
-template <int DT, bool ZP, bool CHANNEL, int TN>
-__global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
+template <int DT, bool ZP, bool CHANNEL, int TN, int DNW>
+__global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   constexpr int W = TN / 32;  // Marlin words per lane and k-tile: 4 (128-bit load) or 2 (64-bit load)
   constexpr bool HI_TRICK = (DT == DT_F16) && !ZP;
   constexpr int RS = DecodeCfg<TN>::RS;
@@ -306,7 +308,9 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   float* red = (float*)smem;
   const int t = threadIdx.x;
   constexpr int CPT = TN / 32;          // consecutive columns per thread in the final phase (4 or 2)
-  const int fr = t >> 5;                // tile row
+  constexpr int RPP = DNW * 2;          // tile rows per pass of the final phase (32 threads per row)
+  constexpr int NP = 16 / RPP;          // passes: thread t has rows (t >> 5) + RPP * pass
+  const int fr0 = t >> 5;
   const int fc = (t & 31) * CPT;        // first column inside the tile
   const int fpos = (TN == 128) ? fc + (fc >= 64 ? 8 : 0) : fc + (fc >= 32 ? 8 : 0);
   const int ncol = ct * TN + fc;
@@ -339,7 +343,7 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   };
   // fused SiLU-and-mul (TN = 128 only, host-checked): the threads of the gate half also take the up half's columns
   const bool act_lane = TN == 128 && p.act && fc < 64;
-  auto finalize = [&](float* v, float* u) {
+  auto finalize = [&](float* v, float* u, int fr) {
     const int crow = s_crow[fr];
     if (crow < 0) return;
     if constexpr (TN == 128) {
@@ -385,30 +389,42 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
         for (int r = 0; r < 4; ++r) mine[(4 * g + r) * RS + HS * h + 16 * w + 8 * hf + c] = acc[w][hf][r];
   }
   __syncthreads();
-  float v[CPT], u[CPT];
+  float v[NP][CPT], u[NP][CPT];
 #pragma unroll
-  for (int j = 0; j < CPT; ++j) v[j] = u[j] = 0.0f;
+  for (int ps = 0; ps < NP; ++ps) {
+    const int fr = fr0 + RPP * ps;
 #pragma unroll
-  for (int ww = 0; ww < DNW; ++ww) {
-    const float* src = red + ww * (16 * RS) + fr * RS + fpos;
+    for (int j = 0; j < CPT; ++j) v[ps][j] = u[ps][j] = 0.0f;
 #pragma unroll
-    for (int j = 0; j < CPT; ++j) v[j] += src[j];
+    for (int ww = 0; ww < DNW; ++ww) {
+      const float* src = red + ww * (16 * RS) + fr * RS + fpos;
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) v[ps][j] += src[j];
+    }
   }
   if (single) {
-    if (act_lane) {
 #pragma unroll
-      for (int ww = 0; ww < DNW; ++ww) {
-        const float* src = red + ww * (16 * RS) + fr * RS + fpos + 72;
+    for (int ps = 0; ps < NP; ++ps) {
+      const int fr = fr0 + RPP * ps;
+      if (act_lane) {
 #pragma unroll
-        for (int j = 0; j < CPT; ++j) u[j] += src[j];
+        for (int ww = 0; ww < DNW; ++ww) {
+          const float* src = red + ww * (16 * RS) + fr * RS + fpos + 72;
+#pragma unroll
+          for (int j = 0; j < CPT; ++j) u[ps][j] += src[j];
+        }
       }
+      finalize(v[ps], u[ps], fr);
     }
-    finalize(v, u);
     return;
   }
-  if (s_crow[fr] >= 0) {
 #pragma unroll
-    for (int j = 0; j < CPT; j += 2) store_coherent2(my_part + fr * TN + fc + j, v[j], v[j + 1]);
+  for (int ps = 0; ps < NP; ++ps) {
+    const int fr = fr0 + RPP * ps;
+    if (s_crow[fr] >= 0) {
+#pragma unroll
+      for (int j = 0; j < CPT; j += 2) store_coherent2(my_part + fr * TN + fc + j, v[ps][j], v[ps][j + 1]);
+    }
   }
   // ---- cross-workgroup reduction: the last split to arrive sums all partials in split order
   __builtin_amdgcn_s_waitcnt(0);
@@ -416,7 +432,10 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
   if (t == 0) s_last = arrive_last(p.locks + tile * p.lock_stride, p.splits);
   __syncthreads();
   if (!s_last) return;
-  if (s_crow[fr] >= 0) {
+#pragma unroll
+  for (int ps = 0; ps < NP; ++ps) {
+    const int fr = fr0 + RPP * ps;
+    if (s_crow[fr] < 0) continue;
     auto sum_parts = [&](float* out, int col) {
       const float* parts = p.ctmp + (int64_t)tile * p.splits * (16 * TN) + fr * TN + col;
 #pragma unroll
@@ -438,40 +457,45 @@ __global__ __launch_bounds__(DNW * 64) void decode_kernel(const KParams p) {
           }
       }
     };
-    sum_parts(v, fc);
-    if (act_lane) sum_parts(u, fc + 64);
-    finalize(v, u);
+    sum_parts(v[ps], fc);
+    if (act_lane) sum_parts(u[ps], fc + 64);
+    finalize(v[ps], u[ps], fr);
   }
 }
 
 // ------------------------------------------------------------------------------------ host side
 typedef void (*decode_fn)(const KParams);
 
+template <int DT, int TN, int NW>
+static decode_fn pick4(bool zp, bool channel) {
+  if (zp) return channel ? decode_kernel<DT, true, true, TN, NW> : decode_kernel<DT, true, false, TN, NW>;
+  return channel ? decode_kernel<DT, false, true, TN, NW> : decode_kernel<DT, false, false, TN, NW>;
+}
 template <int DT, int TN>
-static decode_fn pick3(bool zp, bool channel) {
-  if (zp) return channel ? decode_kernel<DT, true, true, TN> : decode_kernel<DT, true, false, TN>;
-  return channel ? decode_kernel<DT, false, true, TN> : decode_kernel<DT, false, false, TN>;
+static decode_fn pick3(int nw, bool zp, bool channel) {
+  return nw == 4 ? pick4<DT, TN, 4>(zp, channel) : pick4<DT, TN, 8>(zp, channel);
 }
 template <int DT>
-static decode_fn pick2(int tn, bool zp, bool channel) {
-  return tn == 64 ? pick3<DT, 64>(zp, channel) : pick3<DT, 128>(zp, channel);
+static decode_fn pick2(int tn, int nw, bool zp, bool channel) {
+  return tn == 64 ? pick3<DT, 64>(nw, zp, channel) : pick3<DT, 128>(nw, zp, channel);
 }
 
 // (act-order never reaches the kernel as such: the host gathers A's columns in front of the launch, see gemm.hip)
-static decode_fn pick_decode(int dt, int tn, bool zp, bool channel) {
-  return dt == DT_F16 ? pick2<DT_F16>(tn, zp, channel) : pick2<DT_BF16>(tn, zp, channel);
+static decode_fn pick_decode(int dt, int tn, int nw, bool zp, bool channel) {
+  return dt == DT_F16 ? pick2<DT_F16>(tn, nw, zp, channel) : pick2<DT_BF16>(tn, nw, zp, channel);
 }
 
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
   if (pl.use_perm) return fail(W4A16_EINVAL, "unsupported kernel variant");
-  decode_fn fn = pick_decode(a->dtype, pl.tn, zp, pl.gm == GM_CHANNEL);
+  const int nw = pl.nw == 4 ? 4 : 8;
+  decode_fn fn = pick_decode(a->dtype, pl.tn, nw, zp, pl.gm == GM_CHANNEL);
   KParams p = make_kparams(a, pl);
-  const int smem = pl.tn == 64 ? DecodeCfg<64>::SMEM : DecodeCfg<128>::SMEM;
+  const int smem = pl.tn == 64 ? DecodeCfg<64>::smem(nw) : DecodeCfg<128>::smem(nw);
   W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
   const int64_t grid = (int64_t)pl.tiles * pl.splits;
   if (grid <= 0) return 0;
-  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(DNW * 64), smem, stream, p);
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(nw * 64), smem, stream, p);
   W4A16_HIP(hipGetLastError());
   return 0;
 }
