@@ -38,11 +38,19 @@ def default_activation_func(activation: str, output: torch.Tensor, input: torch.
     ops.silu_and_mul(output, input)
 
 
-def pick_block_size(tokens: int, topk: int, num_experts: int) -> int:
-    """Smallest block that the average expert's share of the token slots fills to less than 90 %
-    (the reference's rule, fused_marlin_moe.py:279-282), else the largest."""
+def pick_block_size(tokens: int, topk: int, num_experts: int, expert_bytes: int = 1 << 30) -> int:
+    """Token slots per expert block, from the average expert's share of the slots (the quantity the reference's rule
+    uses, fused_marlin_moe.py:279-282), fitted to the kernels behind each size on MI355X: blocks of 16 slots run on the
+    weight-streaming kernel, whose cost is one pass over the expert's weights per block; blocks of 64 on the 64-row
+    kernel, which costs about two such passes per block, so it wins once an expert fills more than one and a half
+    blocks of 16 (sooner for experts of a few MB, where the per-block fixed costs count).  Blocks of 32 and 48 only pay
+    while there are too few blocks of 64 to give every compute unit work (few, large experts)."""
     per_expert = tokens * topk / num_experts
-    return next((bs for bs in _BLOCK_SIZES if per_expert < 0.9 * bs), _BLOCK_SIZES[-1])
+    if per_expert < (20 if expert_bytes >= (12 << 20) else 14):
+        return 16
+    if num_experts * (per_expert / 64 + 0.5) < 12:
+        return next((bs for bs in (32, 48) if per_expert < 0.9 * bs), 64)
+    return 64
 
 
 @dataclass
@@ -165,7 +173,7 @@ def fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, ga
     _check_layer(k, w1, w2, quant_type, hidden_states.dtype)
     num_local = w1.size(0)
     topk = topk_ids.size(1)
-    bs = pick_block_size(m, topk, num_local)
+    bs = pick_block_size(m, topk, num_local, (w1[0].numel() + w2[0].numel()) * 4)
     sorted_ids, expert_ids, post_pad = moe_align_block_size(
         topk_ids, bs, num_local if global_num_experts == -1 else global_num_experts, expert_map)
     ex = _Experts(quant_type, (w1, w2), (w1_scale, w2_scale), (bias1, bias2), (global_scale1, global_scale2),
