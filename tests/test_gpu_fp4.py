@@ -150,7 +150,8 @@ def test_argument_errors(ops, dev, workspace):
 
 
 @pytest.mark.parametrize("kind,dtype", [("nvfp4", torch.float16), ("nvfp4", torch.bfloat16), ("mxfp4", torch.bfloat16)])
-@pytest.mark.parametrize("m,topk,e,bs", [(3, 2, 4, 8), (123, 2, 4, 32), (333, 2, 4, 64)])
+# (600 tokens in blocks of 8: more 16-row tiles than compute units, the 4-wavefront form of the general kernel)
+@pytest.mark.parametrize("m,topk,e,bs", [(3, 2, 4, 8), (123, 2, 4, 32), (333, 2, 4, 64), (600, 2, 4, 8)])
 def test_moe_gemm_fp4_experts(ops, dev, kind, dtype, m, topk, e, bs):
     """Per-expert weights, scale bytes and (NVFP4) global scales through moe_wna16_marlin_gemm."""
     from oracle import moe_ref as mr

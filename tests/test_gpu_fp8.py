@@ -156,7 +156,8 @@ def test_act_order_is_rejected(ops, dev, workspace):
                              vst.scalar_types.float8_e4m3fn, 4, size_n, size_k)
 
 
-@pytest.mark.parametrize("m,topk,e,bs", [(3, 2, 4, 8), (123, 2, 4, 32), (333, 2, 4, 64)])
+# (600 tokens in blocks of 8: more 16-row tiles than compute units, the 4-wavefront form of the general kernel)
+@pytest.mark.parametrize("m,topk,e,bs", [(3, 2, 4, 8), (123, 2, 4, 32), (333, 2, 4, 64), (600, 2, 4, 8)])
 @pytest.mark.parametrize("dtype,group", [(torch.float16, 128), (torch.bfloat16, -1)])
 def test_moe_gemm_fp8_experts(ops, dev, m, topk, e, bs, dtype, group):
     from oracle import moe_ref as mr

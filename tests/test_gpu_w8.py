@@ -48,6 +48,22 @@ def test_one_hot_rows_are_exact_w8(ops, dev, workspace, dtype, group):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group", [-1, 128])
+def test_wide_layer_more_tiles_than_compute_units_w8(ops, dev, workspace, dtype, group):
+    """N / 128 = 300 column tiles of 16 rows: the general kernel's 4-wavefront form (final phase in two row passes)."""
+    k, n = 128, 128 * 300
+    layer = make_layer(k, n, group, dtype, seed=4, bits=8)
+    ks = torch.randperm(k, generator=torch.Generator().manual_seed(1))[:16]
+    a = torch.zeros(16, k, dtype=dtype)
+    a[torch.arange(16), ks] = 1.0
+    out = run_gemm(ops, layer, a.to(dev), dev, workspace)
+    assert torch.equal(out.cpu(), layer.w_ref[ks])
+    a = torch.randn(5, k, generator=torch.Generator().manual_seed(2)).to(dtype).to(dev)
+    check_close(run_gemm(ops, layer, a, dev, workspace), a, layer)
+    assert int(workspace.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 16, 33, 100, 512])
 @pytest.mark.parametrize("group,act_order,k_full", [(-1, False, True), (128, False, True), (64, True, True), (128, True, False)])
 def test_gemm_w8(ops, dev, workspace, dtype, m, group, act_order, k_full):
@@ -117,7 +133,8 @@ def test_linear_kernel_w8(dev):
     assert mt["max_rel"] <= 2e-2 and mt["mean_rel"] < 0.04, mt
 
 
-@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 4, 8), (33, 2, 8, 16), (123, 3, 4, 32), (333, 2, 4, 64)])
+# (300 tokens in blocks of 8: more 16-row tiles than compute units, the 4-wavefront form of the general kernel)
+@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 4, 8), (33, 2, 8, 16), (123, 3, 4, 32), (333, 2, 4, 64), (300, 4, 4, 8)])
 @pytest.mark.parametrize("dtype,k_full", [(torch.float16, True), (torch.bfloat16, True), (torch.float16, False)])
 def test_moe_gemm_w8_act_order(ops, dev, dtype, k_full, m, topk, e, bs):
     """uint8b128 experts with act-order (per-expert g_idx and column gather inside the kernel), which the reference

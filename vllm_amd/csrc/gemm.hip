@@ -366,8 +366,9 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     pl.kps = kps;
     pl.splits = (int)ceil_div(pl.total_ksteps, kps);
   }
-  // decode kernel: more workgroups than compute units -> 4-wavefront workgroups, two to a compute unit
-  pl.nw = forced_nw ? forced_nw : (pl.kind == 1 && (int64_t)pl.tiles * pl.splits > cus) ? 4 : 8;
+  // 16-row tiles, more workgroups than compute units -> 4-wavefront workgroups, two to a compute unit
+  pl.nw = forced_nw ? forced_nw
+          : ((pl.kind == 1 || (pl.kind == 0 && pl.mb == 1)) && (int64_t)pl.tiles * pl.splits > cus) ? 4 : 8;
   if (debug_plan)
     fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=%d tn=%d mb=%d tiles=%d splits=%d kps=%d nw=%d model_us=%.2f\n",
             (long long)a->size_m, (long long)a->size_n, (long long)a->size_k, pl.kind, pl.tn, pl.mb, pl.tiles,

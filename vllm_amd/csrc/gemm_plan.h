@@ -16,7 +16,7 @@ struct Plan {
   int kind;  // 0: skinny kernel, 1: decode kernel, 2: prefill ("fat") kernel, 3: 64-row ("mid") kernel,
              // 5: 64-row kernel with the in-workgroup K split (gemm_kq.hip)
   int tn;    // tile width in columns (128; the decode kernel also has 64)
-  int nw = 8;  // decode kernel: wavefronts per workgroup (8 or 4)
+  int nw = 8;  // 16-row tiles (decode kernel, general kernel with one m-block): wavefronts per workgroup (8 or 4)
   int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
   int tail_strips = 0; // prefill plan: trailing 512-column strips handed to the 64-row kernel (0 = none)
   int64_t ctmp_bytes;  // fp32 split-K partials

@@ -29,19 +29,22 @@
 
 namespace w4a16 {
 
-constexpr int NW = 8;        // wavefronts per workgroup
+// Wavefronts per workgroup (template parameter NW): 8; one-m-block tiles also come with 4, for launches with more
+// workgroups than compute units, where two 4-wavefront workgroups share a compute unit and each one's prologue and
+// epilogue run under the other's weight stream.
 
 template <int MB>
 struct SkinnyCfg {
   // k-steps in flight per wavefront (measured: deeper rings on the taller tiles cost registers, hence spills, and time)
   static constexpr int D = (MB >= 4) ? 2 : (MB == 2) ? 4 : 6;
-  static constexpr int SMEM = NW * 16 * RED_RS * 4;  // reduction slab; its head doubles as the A bounce slabs
+  static constexpr int smem(int nw) { return nw * 16 * RED_RS * 4; }  // reduction slab; its head doubles as the A bounce slabs
 };
 
 
 // FP4: 0 = integer weights, 1 = float4_e2m1f with NVFP4 scales (per k-tile), 2 = with MXFP4 scales (per k-step)
-template <int DT, int MB, bool ZP, int GM, int BITS = 4, bool ZPF = false, bool FP8 = false, int FP4 = 0>
-__global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
+template <int DT, int MB, bool ZP, int GM, int BITS = 4, bool ZPF = false, bool FP8 = false, int FP4 = 0, int NW = 8>
+__global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
+  static_assert(NW == 8 || (NW == 4 && MB == 1), "4-wavefront workgroups: one-m-block tiles only");
   static_assert(BITS == 4 || (BITS == 8 && !ZP), "8-bit weights are uint8b128 (no zero points)");
   // ZPF: fp16 zero points laid out like the scales (HQQ); element-wise dequantisation on every tile size
   static_assert(FP4 == 0 || (BITS == 4 && !ZP && !ZPF && GM == GM_GROUPED), "fp4 weights: grouped scale records");
@@ -454,7 +457,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
   // store hit 64 distinct banks: c + 8h + 16*(row/4).
   float* red = (float*)smem;
   const int t = threadIdx.x;
-  const int fr = t >> 5;            // 0..15: tile row handled in the final phase
+  constexpr int RPP = NW * 2;       // tile rows per pass of the final phase (32 threads per row)
+  const int fr0 = t >> 5;           // 0..RPP-1: tile row handled in the first pass
   const int fc4 = (t & 31) * 4;     // first of 4 consecutive columns inside the column pair
   const int fpos = fc4 + (fc4 >= 64 ? 8 : 0);
   const int ncol = cp * 128 + fc4;  // real column
@@ -522,19 +526,23 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
             mine[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
     }
     __syncthreads();
-    f32x4 v = *(const f32x4*)(red + fr * RED_RS + fpos);
 #pragma unroll
-    for (int ww = 1; ww < NW; ++ww) v += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos);
-    const int r = mb * 16 + fr;
-    if (single) {
-      f32x4 u = {0, 0, 0, 0};
-      if (act_lane) {
+    for (int ps = 0; ps < 16 / RPP; ++ps) {
+      const int fr = fr0 + ps * RPP;
+      f32x4 v = *(const f32x4*)(red + fr * RED_RS + fpos);
 #pragma unroll
-        for (int ww = 0; ww < NW; ++ww) u += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos + 72);
+      for (int ww = 1; ww < NW; ++ww) v += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos);
+      const int r = mb * 16 + fr;
+      if (single) {
+        f32x4 u = {0, 0, 0, 0};
+        if (act_lane) {
+#pragma unroll
+          for (int ww = 0; ww < NW; ++ww) u += *(const f32x4*)(red + ww * (16 * RED_RS) + fr * RED_RS + fpos + 72);
+        }
+        finalize(r, v, u);
+      } else if (s_crow[r] >= 0) {
+        store_coherent(my_part + r * 128 + fc4, v);
       }
-      finalize(r, v, u);
-    } else if (s_crow[r] >= 0) {
-      store_coherent(my_part + r * 128 + fc4, v);
     }
   }
   if (single) return;
@@ -562,7 +570,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
     return v;
   };
 #pragma unroll 1
-  for (int r = fr; r < BM; r += 16) {
+  for (int r = fr0; r < BM; r += RPP) {
     if (s_crow[r] < 0) continue;
     const f32x4 v = sum_parts(r, fc4);
     f32x4 u = {0, 0, 0, 0};
@@ -574,56 +582,61 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const KParams p) {
 // ------------------------------------------------------------------------------------ host side
 typedef void (*skinny_fn)(const KParams);
 
-template <int DT, int MB>
+template <int DT, int MB, int NW = 8>
 static skinny_fn pick_zp_gm(bool zp, int gm) {
   if (zp) {
-    if (gm == GM_GROUPED) return skinny_kernel<DT, MB, true, GM_GROUPED>;
-    if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, true, GM_CHANNEL>;
+    if (gm == GM_GROUPED) return skinny_kernel<DT, MB, true, GM_GROUPED, 4, false, false, 0, NW>;
+    if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, true, GM_CHANNEL, 4, false, false, 0, NW>;
     return nullptr;
   }
-  if (gm == GM_GROUPED) return skinny_kernel<DT, MB, false, GM_GROUPED>;
-  if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, false, GM_CHANNEL>;
-  return skinny_kernel<DT, MB, false, GM_GIDX>;
+  if (gm == GM_GROUPED) return skinny_kernel<DT, MB, false, GM_GROUPED, 4, false, false, 0, NW>;
+  if (gm == GM_CHANNEL) return skinny_kernel<DT, MB, false, GM_CHANNEL, 4, false, false, 0, NW>;
+  return skinny_kernel<DT, MB, false, GM_GIDX, 4, false, false, 0, NW>;
 }
 
+// (nw = 4 exists for one-m-block tiles only; the planner asks for it nowhere else)
 template <int DT>
-static skinny_fn pick_mb(int mb, bool zp, int gm) {
+static skinny_fn pick_mb(int mb, int nw, bool zp, int gm) {
   switch (mb) {
-    case 1: return pick_zp_gm<DT, 1>(zp, gm);
+    case 1: return nw == 4 ? pick_zp_gm<DT, 1, 4>(zp, gm) : pick_zp_gm<DT, 1>(zp, gm);
     case 2: return pick_zp_gm<DT, 2>(zp, gm);
     default: return pick_zp_gm<DT, 4>(zp, gm);
   }
 }
 
-template <int DT, int MB>
+template <int DT, int MB, int NW = 8>
 static skinny_fn pick_w8_gm(int gm) {  // uint8b128: no zero points
-  return gm == GM_GROUPED ? skinny_kernel<DT, MB, false, GM_GROUPED, 8>
-         : gm == GM_CHANNEL ? skinny_kernel<DT, MB, false, GM_CHANNEL, 8>
-                            : skinny_kernel<DT, MB, false, GM_GIDX, 8>;
+  return gm == GM_GROUPED ? skinny_kernel<DT, MB, false, GM_GROUPED, 8, false, false, 0, NW>
+         : gm == GM_CHANNEL ? skinny_kernel<DT, MB, false, GM_CHANNEL, 8, false, false, 0, NW>
+                            : skinny_kernel<DT, MB, false, GM_GIDX, 8, false, false, 0, NW>;
 }
 
 template <int DT>
-static skinny_fn pick_w8(int mb, int gm) {
-  return mb == 1 ? pick_w8_gm<DT, 1>(gm) : mb == 2 ? pick_w8_gm<DT, 2>(gm) : pick_w8_gm<DT, 4>(gm);
+static skinny_fn pick_w8(int mb, int nw, int gm) {
+  return mb == 1 ? (nw == 4 ? pick_w8_gm<DT, 1, 4>(gm) : pick_w8_gm<DT, 1>(gm))
+         : mb == 2 ? pick_w8_gm<DT, 2>(gm) : pick_w8_gm<DT, 4>(gm);
 }
 
 // (act-order never reaches a kernel as such: the host gathers A's columns in front of the launch, see gemm.hip)
-static skinny_fn pick_skinny(int dt, int mb, bool zp, int gm, bool w8) {
+static skinny_fn pick_skinny(int dt, int mb, int nw, bool zp, int gm, bool w8) {
   if (w8) {
     if (zp) return nullptr;
-    return dt == DT_F16 ? pick_w8<DT_F16>(mb, gm) : pick_w8<DT_BF16>(mb, gm);
+    return dt == DT_F16 ? pick_w8<DT_F16>(mb, nw, gm) : pick_w8<DT_BF16>(mb, nw, gm);
   }
-  return dt == DT_F16 ? pick_mb<DT_F16>(mb, zp, gm) : pick_mb<DT_BF16>(mb, zp, gm);
+  return dt == DT_F16 ? pick_mb<DT_F16>(mb, nw, zp, gm) : pick_mb<DT_BF16>(mb, nw, zp, gm);
 }
 
-static int skinny_smem_bytes(int mb) {
-  return mb == 1 ? SkinnyCfg<1>::SMEM : mb == 2 ? SkinnyCfg<2>::SMEM : SkinnyCfg<4>::SMEM;
+static int skinny_smem_bytes(int mb, int nw) {
+  return mb == 1 ? SkinnyCfg<1>::smem(nw) : mb == 2 ? SkinnyCfg<2>::smem(nw) : SkinnyCfg<4>::smem(nw);
 }
 
 template <int DT>
-static skinny_fn pick_fp8(int mb, int gm) {  // float8_e4m3fn: grouped or channel-wise scales, no act-order
+static skinny_fn pick_fp8(int mb, int nw, int gm) {  // float8_e4m3fn: grouped or channel-wise scales, no act-order
   switch (mb) {
     case 1:
+      if (nw == 4)
+        return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, 8, false, true, 0, 4>
+                                : skinny_kernel<DT, 1, false, GM_CHANNEL, 8, false, true, 0, 4>;
       return gm == GM_GROUPED ? skinny_kernel<DT, 1, false, GM_GROUPED, 8, false, true>
                               : skinny_kernel<DT, 1, false, GM_CHANNEL, 8, false, true>;
     case 2:
@@ -636,17 +649,21 @@ static skinny_fn pick_fp8(int mb, int gm) {  // float8_e4m3fn: grouped or channe
 }
 
 template <int DT, int FP4>
-static skinny_fn pick_fp4(int mb) {  // float4_e2m1f (validated on the host: grouped records, no act-order, dense)
+static skinny_fn pick_fp4(int mb, int nw) {  // float4_e2m1f (validated on the host: grouped records, no act-order)
   switch (mb) {
-    case 1: return skinny_kernel<DT, 1, false, GM_GROUPED, 4, false, false, FP4>;
+    case 1:
+      return nw == 4 ? skinny_kernel<DT, 1, false, GM_GROUPED, 4, false, false, FP4, 4>
+                     : skinny_kernel<DT, 1, false, GM_GROUPED, 4, false, false, FP4>;
     case 2: return skinny_kernel<DT, 2, false, GM_GROUPED, 4, false, false, FP4>;
     default: return skinny_kernel<DT, 4, false, GM_GROUPED, 4, false, false, FP4>;
   }
 }
 
-static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
+static skinny_fn pick_zpf(int mb, int nw) {  // fp16 zero points (validated on the host: fp16, uint4, grouped, no act-order)
   switch (mb) {
-    case 1: return skinny_kernel<DT_F16, 1, false, GM_GROUPED, 4, true>;
+    case 1:
+      return nw == 4 ? skinny_kernel<DT_F16, 1, false, GM_GROUPED, 4, true, false, 0, 4>
+                     : skinny_kernel<DT_F16, 1, false, GM_GROUPED, 4, true>;
     case 2: return skinny_kernel<DT_F16, 2, false, GM_GROUPED, 4, true>;
     default: return skinny_kernel<DT_F16, 4, false, GM_GROUPED, 4, true>;
   }
@@ -654,25 +671,26 @@ static skinny_fn pick_zpf(int mb) {  // fp16 zero points (validated on the host:
 
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
+  const int nw = (pl.nw == 4 && pl.mb == 1) ? 4 : 8;
   skinny_fn fn;
   if (a->flags & W4A16_F_ZP_FLOAT)
-    fn = pick_zpf(pl.mb);
+    fn = pick_zpf(pl.mb, nw);
   else if (a->wtype == W4A16_WTYPE_FE2M1)
-    fn = a->global_scale ? (a->dtype == DT_F16 ? pick_fp4<DT_F16, 1>(pl.mb) : pick_fp4<DT_BF16, 1>(pl.mb))
-                         : pick_fp4<DT_BF16, 2>(pl.mb);
+    fn = a->global_scale ? (a->dtype == DT_F16 ? pick_fp4<DT_F16, 1>(pl.mb, nw) : pick_fp4<DT_BF16, 1>(pl.mb, nw))
+                         : pick_fp4<DT_BF16, 2>(pl.mb, nw);
   else if (a->wtype == W4A16_WTYPE_FE4M3)
     fn = pl.gm == GM_GIDX     ? nullptr
-         : a->dtype == DT_F16 ? pick_fp8<DT_F16>(pl.mb, pl.gm)
-                              : pick_fp8<DT_BF16>(pl.mb, pl.gm);
+         : a->dtype == DT_F16 ? pick_fp8<DT_F16>(pl.mb, nw, pl.gm)
+                              : pick_fp8<DT_BF16>(pl.mb, nw, pl.gm);
   else
-    fn = pick_skinny(a->dtype, pl.mb, zp, pl.gm, a->wtype == W4A16_WTYPE_U8B128);
+    fn = pick_skinny(a->dtype, pl.mb, nw, zp, pl.gm, a->wtype == W4A16_WTYPE_U8B128);
   if (!fn || pl.use_perm) return fail(W4A16_EINVAL, "unsupported kernel variant");
   KParams p = make_kparams(a, pl);
-  const int smem = skinny_smem_bytes(pl.mb);
+  const int smem = skinny_smem_bytes(pl.mb, nw);
   W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
   const int64_t grid = (int64_t)pl.tiles * pl.splits;
   if (grid <= 0) return 0;
-  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(NW * 64), smem, stream, p);
+  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(nw * 64), smem, stream, p);
   W4A16_HIP(hipGetLastError());
   return 0;
 }
