@@ -248,3 +248,16 @@ def test_mixtral_moe_gemm_one_hot(dev, mixtral, which):
             use_fp32_reduce=True, is_zp_float=False).cpu()
         for (tok, slot), row in want.items():
             assert torch.equal(out[tok * topk + slot], row), (bs, tok, slot)
+
+
+@pytest.mark.parametrize("m", [192, 320, 512, 768, 1024])
+@pytest.mark.parametrize("kind", ["gptq_f16", "awq_bf16"])
+@pytest.mark.parametrize("name", ["qkv", "o", "down"])
+def test_narrow_layers_between_decode_and_prefill(dev, ws, name, kind, m):
+    """129..1024 rows on the layers too narrow for the prefill kernel: the planner moves between the general kernel,
+    64 x 256 tiles with the K range cut inside the workgroup (and, for down_proj's long K, across workgroups with a
+    second pass over the partial tiles) and the 64 x 512 kernel."""
+    print(f"narrow layer {kind} {name} m={m}", flush=True)
+    L = _layer(kind, name, dev)
+    _check_one_hot(L, m, ws, dev)
+    _check_random(L, m, ws, dev)

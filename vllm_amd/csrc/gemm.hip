@@ -220,7 +220,21 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     // give between 3/4 and all of the compute units a workgroup (4096 x 28672: 45 / 44 us at 96 / 128 rows against
     // 54 / 58; 8192 x 57344: 75-82 us at 33-64 rows against 87-101), level at 1.75 rounds, behind with fewer tiles
     const int64_t kq_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 256);
-    const bool kq_pays = a->size_m <= 128 && kq_tiles >= cus * 3 / 4 && kq_tiles <= cus;
+    // Above 128 rows (layers too narrow for the prefill kernel's 128 x 512 tiles): against the 64 x 512 kernel these
+    // tiles win whenever they fit one round (4096 x 4096 at 1024 rows: 44 against 59 us); against the general kernel's
+    // 64 x 128 tiles once those need a second round (4096 x 6144 at 384 rows: 38 against 50 us).  With a long K and
+    // few tiles, K is also split across workgroups while every wavefront keeps at least 24 k-steps (14336 x 4096 at
+    // 192..512 rows: 5-9 % ahead of the general kernel; with shorter splits the fixed costs of the two launches win).
+    int kq_sp = 1;
+    const int64_t gen_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 128);
+    const bool kq_tall = a->size_m > 128 && kq_tiles <= cus;
+    if (kq_tall)
+      while (kq_sp < 8 && kq_tiles * kq_sp * 2 <= cus && pl.total_ksteps % (32 * kq_sp) == 0 &&
+             pl.total_ksteps / (8 * kq_sp) >= 24)
+        kq_sp *= 2;
+    if (forced_splits > 0 && forced_kind == 5 && pl.total_ksteps % (16 * forced_splits) == 0) kq_sp = forced_splits;
+    const bool kq_pays = (a->size_m <= 128 && kq_tiles >= cus * 3 / 4 && kq_tiles <= cus) ||
+                         (kq_tall && kq_tiles * kq_sp >= cus / 2 && (kq_sp > 1 || gen_tiles > cus));
     if (kq_shape && (forced_kind == 5 || (forced_kind < 0 && kq_pays))) {
       pl.kind = 5;
       pl.tn = 256;
@@ -229,12 +243,12 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       pl.mtiles = (int)ceil_div(a->size_m, 64);
       pl.ncp = (int)ceil_div(a->size_n, 256);
       const int64_t tiles = (int64_t)pl.mtiles * pl.ncp;
-      W4A16_CHECK(tiles < (1LL << 31) / 64, "too many tiles");
+      W4A16_CHECK(tiles * kq_sp < (1LL << 31) / 64, "too many tiles");
       pl.tiles = (int)tiles;
-      pl.splits = 1;
-      pl.kps = pl.total_ksteps;
+      pl.splits = kq_sp;
+      pl.kps = pl.total_ksteps / kq_sp;
       pl.xcd_map = 0;
-      pl.ctmp_bytes = 0;
+      pl.ctmp_bytes = kq_sp > 1 ? tiles * kq_sp * 64 * 256 * 4 : 0;
       if (debug_plan)
         fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=5 tiles=%d splits=%d kps=%d\n", (long long)a->size_m,
                 (long long)a->size_n, (long long)a->size_k, pl.tiles, pl.splits, pl.kps);

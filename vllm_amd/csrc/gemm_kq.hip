@@ -10,8 +10,11 @@
 //   activations  each K-quarter stages its own 64 rows x 64 K chunk into LDS in MFMA fragment order (its two
 //                wavefronts share it), double buffered; one workgroup barrier per two k-steps.
 //   epilogue     the four quarters' partial tiles are added through LDS, one 16-row block at a time.
-//   No split across workgroups: the planner only picks this kernel when its tiles about fill the chip (with too few
-//   tiles the partial tiles in HBM and the second launch cost more than the 16-row tiles they would replace).
+//   split-K      with fewer tiles than compute units (129..~1000 rows of a narrow layer) K is also cut across
+//                workgroups, in splits of whole multiples of 512 K rows: the workgroup writes its 64 x 256 fp32 partial
+//                tile (already summed over its quarters) to scratch with plain 128-bit stores and kq_reduce_kernel,
+//                launched right behind, adds the splits in order and finishes the rows.  A quarter of the 64 x 512
+//                kernel's partial bytes for the same number of wavefronts on the problem.
 // Compared with 16-row tiles (which re-read and re-convert the weight strip once per 16 rows) every weight is fetched
 // and dequantised once per 64 rows; compared with the 64 x 512 tile there are 2 x 4 times as many independent streams.
 // Requirements (host-checked): K % 512 == 0 (every quarter runs whole ring periods of 4 k-steps), scales grouped (a
@@ -46,7 +49,7 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
   const int mtiles = (p.M + KQ_BM - 1) / KQ_BM;
   const int mt = blockIdx.x % mtiles;
-  const int strip = blockIdx.x / mtiles;
+  const int split = (blockIdx.x / mtiles) % p.splits, strip = blockIdx.x / (mtiles * p.splits);
   const int cp = strip * 2 + wn;               // column pair of this wavefront
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 256: the trailing wavefronts only help staging
   const int row0 = mt * KQ_BM;
@@ -75,8 +78,8 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
 
   // ---- this quarter's k-steps: [ks_b, ks_e), a multiple of 4 long
-  const int per_q = p.total_ksteps / KQ_Q;  // host: a multiple of 4
-  const int ks_b = q * per_q, ks_e = ks_b + per_q;
+  const int per_q = p.ksteps_per_split / KQ_Q;  // host: a multiple of 4, and the splits are equally long
+  const int ks_b = split * p.ksteps_per_split + q * per_q, ks_e = ks_b + per_q;
 
   // ---- activation staging: the quarter's 128 threads; thread tq loads piece (tq & 7) of tile rows (tq >> 3) + 16 i
   // (rows without a source read row 0 of A; their results are never stored)
@@ -265,7 +268,11 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
       f32x4 v = {0, 0, 0, 0};
 #pragma unroll
       for (int qq = 0; qq < KQ_Q; ++qq) v += *(const f32x4*)(slabs + (qq * 2 + wn) * (16 * RED_RS) + r16 * RED_RS + fpos);
-      if (fcol_ok && crow >= 0) {
+      if (p.splits > 1) {
+        if (crow >= 0)
+          *(f32x4*)(p.ctmp + (((int64_t)(strip * mtiles + mt) * p.splits + split) * KQ_BM + mb * 16 + r16) * KQ_TN +
+                    wn * 128 + fc4) = v;
+      } else if (fcol_ok && crow >= 0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
         u32x2 o;
@@ -280,6 +287,53 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   }
 }
 
+// Second pass of a split-K launch: adds the splits' partial tiles in split order, then channel scale, bias and
+// conversion as kq_kernel's own epilogue.  One workgroup per (tile, 16-row block); thread -> 4 columns of 4 rows.
+template <int DT, bool CHANNEL>
+__global__ __launch_bounds__(256) void kq_reduce_kernel(const KParams p) {
+  const int t = threadIdx.x;
+  const int mtiles = (p.M + KQ_BM - 1) / KQ_BM;
+  const int tile = blockIdx.x >> 2, rb = blockIdx.x & 3;
+  const int mt = tile % mtiles, strip = tile / mtiles;
+  const int fc4 = (t & 63) * 4;
+  const int ncol = strip * KQ_TN + fc4;
+  if (ncol >= p.N) return;
+  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint16_t* bias = (const uint16_t*)p.bias;
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+  {
+    const int base = ncol & ~31, cl = ncol & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        cs[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bs[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  }
+  const float* parts = p.ctmp + (int64_t)tile * p.splits * (KQ_BM * KQ_TN) + fc4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = rb * 16 + (t >> 6) + 4 * i;
+    const int crow = mt * KQ_BM + r;
+    if (crow >= p.M) continue;
+    f32x4 v = {0, 0, 0, 0};
+    for (int sidx = 0; sidx < p.splits; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * KQ_BM + r) * KQ_TN);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
+    u32x2 o;
+    if constexpr (DT == DT_F16)
+      o = u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+    else
+      o = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+    *(u32x2*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+  }
+}
+
 typedef void (*kq_fn)(const KParams);
 
 template <int DT>
@@ -291,14 +345,21 @@ static kq_fn pick_kq(bool zp, bool channel) {
 int launch_kq(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
   if ((a->wtype != W4A16_WTYPE_U4B8 && a->wtype != W4A16_WTYPE_U4) || (a->flags & (W4A16_F_ZP_FLOAT | W4A16_F_MOE)) ||
-      pl.gm == GM_GIDX || pl.use_perm || a->size_k % 512 != 0 || pl.splits != 1 || pl.tn != KQ_TN)
+      pl.gm == GM_GIDX || pl.use_perm || pl.splits < 1 || pl.kps * pl.splits != pl.total_ksteps || pl.kps % 16 != 0 ||
+      pl.tn != KQ_TN)
     return fail(W4A16_EINVAL, "unsupported kernel variant");
   const kq_fn fn = a->dtype == DT_F16 ? pick_kq<DT_F16>(zp, channel) : pick_kq<DT_BF16>(zp, channel);
   KParams p = make_kparams(a, pl);
   if (pl.tiles <= 0) return 0;
   W4A16_HIP(allow_dynamic_lds((const void*)fn, KQ_SMEM));
-  hipLaunchKernelGGL(fn, dim3((unsigned)pl.tiles), dim3(512), KQ_SMEM, stream, p);
+  hipLaunchKernelGGL(fn, dim3((unsigned)((int64_t)pl.tiles * pl.splits)), dim3(512), KQ_SMEM, stream, p);
   W4A16_HIP(hipGetLastError());
+  if (pl.splits > 1) {
+    const kq_fn red = a->dtype == DT_F16 ? (channel ? kq_reduce_kernel<DT_F16, true> : kq_reduce_kernel<DT_F16, false>)
+                                         : (channel ? kq_reduce_kernel<DT_BF16, true> : kq_reduce_kernel<DT_BF16, false>);
+    hipLaunchKernelGGL(red, dim3((unsigned)pl.tiles * 4), dim3(256), 0, stream, p);
+    W4A16_HIP(hipGetLastError());
+  }
   return 0;
 }
 
