@@ -67,51 +67,61 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint32_t* Zp = p.Z;
   const uint16_t* bias = (const uint16_t*)p.bias;
+  // activation loads: lane -> row (lane >> 3) [+ 8 for the second load], 16-byte piece (lane & 7) of the
+  // stage's 128 bytes.  Rows past the end of the problem read the tile's first row; never stored.
+  const int ar = lane >> 3, ap = lane & 7;
+  const int tr = threadIdx.x & 15;
+  // MoE: slot ids of tile rows 0, ar, ar + 8 and tr (clamped into the block; checked against the block size below), the
+  // block's expert and the number of live slots, all loaded together: a workgroup then waits for one round trip, not
+  // five in a row, before it can address its weights and activations (short-K expert GEMMs live only a few of them)
+  int id_0 = 0, id_a0 = 0, id_a1 = 0, id_t = 0, moe_e = 0, moe_ntp = 0;
   if (p.moe) {
-    if (mt * p.moe_bs >= *p.ntpp) return;
-    const int e = p.expert_ids[mt];
-    if (e < 0) return;
-    Bq += e * p.b_estride;
-    Sc += e * p.s_estride;
-    if (ZP) Zp += e * p.z_estride;
-    if (bias) bias += e * p.n_estride;
+    const int* ids = p.sorted_ids + mt * p.moe_bs;
+    const int last = p.moe_bs - 1;
+    id_0 = ids[0];
+    id_a0 = ids[min(ar, last)];
+    id_a1 = ids[min(ar + 8, last)];
+    id_t = ids[min(tr, last)];
+    moe_ntp = *p.ntpp;
+    moe_e = p.expert_ids[mt];
   }
-
-  auto tile_row_ids = [&](int r, int& src, int& dst) {
+  // which A row feeds tile row r and which C row receives it (-1: none); id: the row's slot id (MoE)
+  auto tile_row_ids = [&](int r, int id, int& src, int& dst) {
     src = -1;
     dst = -1;
     if (p.moe) {
-      if (r < p.moe_bs) {
-        const int id = p.sorted_ids[mt * p.moe_bs + r];
-        if ((unsigned)id < (unsigned)p.c_rows) {
-          src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
-          dst = id;
-        }
+      if (r < p.moe_bs && (unsigned)id < (unsigned)p.c_rows) {
+        src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
+        dst = id;
       }
     } else {
       const int gr = mt * 16 + r;
       if (gr < p.M) src = dst = gr;
     }
   };
-  // activation loads: lane -> row (lane >> 3) [+ 8 for the second load], 16-byte piece (lane & 7) of the
-  // stage's 128 bytes.  Rows past the end of the problem read the tile's first row; never stored.
-  const int ar = lane >> 3, ap = lane & 7;
   const uint16_t* arow[2];
   {
     int src0, dst0;
-    tile_row_ids(0, src0, dst0);
+    tile_row_ids(0, id_0, src0, dst0);
     if (src0 < 0) src0 = 0;  // a block whose first slot is padding still reads inside A
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       int src, dst;
-      tile_row_ids(ar + 8 * i, src, dst);
+      tile_row_ids(ar + 8 * i, i ? id_a1 : id_a0, src, dst);
       arow[i] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + ap * 8;
     }
   }
   if (threadIdx.x < 16) {
     int src, dst;
-    tile_row_ids(threadIdx.x, src, dst);
-    s_crow[threadIdx.x] = dst;
+    tile_row_ids(tr, id_t, src, dst);
+    s_crow[tr] = dst;
+  }
+  if (p.moe) {
+    if (mt * p.moe_bs >= moe_ntp || moe_e < 0) return;
+    Bq += moe_e * p.b_estride;
+    Sc += moe_e * p.s_estride;
+    if (ZP) Zp += moe_e * p.z_estride;
+    if (bias) bias += moe_e * p.n_estride;
   }
 
   // ---- this wavefront's stages (pairs of k-steps)

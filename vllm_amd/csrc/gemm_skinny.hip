@@ -96,31 +96,34 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
   const int32_t* gidx = p.gidx;
   const uint16_t* bias = (const uint16_t*)p.bias;
   const uint16_t* gscale = (const uint16_t*)p.gscale;
+  // MoE: slot ids of tile rows 0, 16 mb + am and (threadIdx.x % BM) (clamped into the block; checked against the block
+  // size below), the block's expert and the number of live slots, all loaded together: one round trip, not several in a
+  // row, before the workgroup can address its weights and activations
+  const int tr = threadIdx.x < BM ? threadIdx.x : 0;
+  int id_0 = 0, id_t = 0, id_a[MB], moe_e = 0, moe_ntp = 0;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) id_a[mb] = 0;
   if (p.moe) {
-    if (mt * p.moe_bs >= *p.ntpp) return;
-    const int e = p.expert_ids[mt];
-    if (e < 0) return;
-    Bq += e * p.b_estride;
-    Sc += e * p.s_estride;
-    if (FP4 == 1) gscale += e;
-    if (ZP) Zp += e * p.z_estride;
-    if (gidx) gidx += e * p.k_estride;
-    if (bias) bias += e * p.n_estride;
+    const int* ids = p.sorted_ids + mt * p.moe_bs;
+    const int last = p.moe_bs - 1;
+    id_0 = ids[0];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) id_a[mb] = ids[min(mb * 16 + am, last)];
+    id_t = ids[min(tr, last)];
+    moe_ntp = *p.ntpp;
+    moe_e = p.expert_ids[mt];
   }
 
   // ---- which A row feeds each tile row, which C row it is written to.  Rows past the end of the
   // problem read the tile's first row (always valid) so that LDS never holds uninitialised data;
-  // their results are never stored.
-  auto tile_row_ids = [&](int r, int& src, int& dst) {
+  // their results are never stored.  id: the row's slot id (MoE).
+  auto tile_row_ids = [&](int r, int id, int& src, int& dst) {
     src = -1;
     dst = -1;
     if (p.moe) {
-      if (r < p.moe_bs) {
-        const int id = p.sorted_ids[mt * p.moe_bs + r];
-        if ((unsigned)id < (unsigned)p.c_rows) {
-          src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
-          dst = id;
-        }
+      if (r < p.moe_bs && (unsigned)id < (unsigned)p.c_rows) {
+        src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
+        dst = id;
       }
     } else {
       const int gr = mt * BM + r;
@@ -130,19 +133,28 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
   const uint16_t* arow[MB];
   {
     int src0, dst0;
-    tile_row_ids(0, src0, dst0);
+    tile_row_ids(0, id_0, src0, dst0);
     if (src0 < 0) src0 = 0;  // a block whose first slot is padding still reads inside A
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       int src, dst;
-      tile_row_ids(mb * 16 + am, src, dst);
+      tile_row_ids(mb * 16 + am, id_a[mb], src, dst);
       arow[mb] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + ap * 8;
     }
   }
   if (threadIdx.x < BM) {
     int src, dst;
-    tile_row_ids(threadIdx.x, src, dst);
-    s_crow[threadIdx.x] = dst;
+    tile_row_ids(tr, id_t, src, dst);
+    s_crow[tr] = dst;
+  }
+  if (p.moe) {
+    if (mt * p.moe_bs >= moe_ntp || moe_e < 0) return;
+    Bq += moe_e * p.b_estride;
+    Sc += moe_e * p.s_estride;
+    if (FP4 == 1) gscale += moe_e;
+    if (ZP) Zp += moe_e * p.z_estride;
+    if (gidx) gidx += moe_e * p.k_estride;
+    if (bias) bias += moe_e * p.n_estride;
   }
 
   // ---- this wavefront's k-steps
