@@ -241,6 +241,29 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_sliced_kernel(
   }
 }
 
+// B terms' loads in flight together (a few tokens give too few wavefronts to hide one round trip per term); added in
+// term order
+template <int DT, int B>
+__device__ __forceinline__ void moe_sum_terms(const uint16_t* __restrict__ in, int64_t tok, int top_k, int64_t hidden8,
+                                              int64_t col, float* acc) {
+  for (int k0 = 0; k0 < top_k; k0 += B) {
+    u32x4 v[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i)
+      v[i] = *(const u32x4*)(in + ((tok * top_k + min(k0 + i, top_k - 1)) * hidden8 + col) * 8);
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      if (k0 + i < top_k) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] += DT == DT_F16 ? f16_lo_f32(v[i][j]) : bf16_lo_f32(v[i][j]);
+          acc[2 * j + 1] += DT == DT_F16 ? f16_hi_f32(v[i][j]) : bf16_hi_f32(v[i][j]);
+        }
+      }
+    }
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
                                                       int64_t total8, int top_k, int64_t hidden8) {
@@ -248,14 +271,12 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t* __restrict
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total8; idx += (int64_t)gridDim.x * 256) {
     const int64_t tok = idx / hidden8, col = idx % hidden8;
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k = 0; k < top_k; ++k) {
-      const u32x4 v = *(const u32x4*)(in + ((tok * top_k + k) * hidden8 + col) * 8);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[2 * j] += DT == DT_F16 ? f16_lo_f32(v[j]) : bf16_lo_f32(v[j]);
-        acc[2 * j + 1] += DT == DT_F16 ? f16_hi_f32(v[j]) : bf16_hi_f32(v[j]);
-      }
-    }
+    if (top_k <= 2)
+      moe_sum_terms<DT, 2>(in, tok, top_k, hidden8, col, acc);
+    else if (top_k <= 4)
+      moe_sum_terms<DT, 4>(in, tok, top_k, hidden8, col, acc);
+    else
+      moe_sum_terms<DT, 8>(in, tok, top_k, hidden8, col, acc);
     u32x4 o;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
