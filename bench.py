@@ -395,6 +395,9 @@ def main():
     ap.add_argument("--probe-shape", type=str, default="",
                     help="counter-collection workload for one shape, LAYER:M:KIND with KIND gptq_f16 or awq_bf16 "
                          "(e.g. gate_up:4096:awq_bf16): a few eager launches on rotating weight copies; prints no JSON line")
+    ap.add_argument("--probe-moe", type=int, default=0, metavar="T",
+                    help="kernel-trace workload: ten calls of the Mixtral-8x7B-shaped fused MoE (8 experts, top-2, uint4b8 "
+                         "g128 fp16, random codes) on T tokens; prints no JSON line")
     ap.add_argument("--issue-probe", action="store_true",
                     help="MFMA / VALU issue micro-benchmark (independent MFMAs interleaved with 0..6 VALU instructions, "
                          "one and two wavefronts per SIMD); prints a table, no JSON line")
@@ -424,6 +427,24 @@ def main():
     if args.stream_probe:
         from vllm_amd import issue_probe
         issue_probe.stream_floor(dev, LAYERS, time_graph, copies_needed)
+        return
+    if args.probe_moe:
+        from vllm_amd.fused_marlin_moe import fused_marlin_moe
+        e, hid, inter, topk, t = 8, 4096, 14336, 2, args.probe_moe
+        gen = torch.Generator(device=dev).manual_seed(3)
+        codes = lambda *shape: torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device=dev, generator=gen)
+        scales = lambda *shape: (torch.rand(shape, device=dev, generator=gen) * 0.01 + 0.001).half()
+        q1, s1 = codes(e, hid // 16, 2 * inter * 2), scales(e, hid // GROUP, 2 * inter)
+        q2, s2 = codes(e, inter // 16, hid * 2), scales(e, inter // GROUP, hid)
+        x = (torch.randn(t, hid, device=dev, generator=gen) / 10).half()
+        logits = torch.randn(t, e, device=dev, generator=gen)
+        tw, ti = torch.topk(torch.softmax(logits, dim=-1), topk)
+        tw, ti = (tw / tw.sum(dim=-1, keepdim=True)).contiguous(), ti.to(torch.int32).contiguous()
+        for _ in range(10):
+            fused_marlin_moe(x, q1, q2, None, None, s1, s2, logits, tw, ti, quant_type_id=scalar_types.uint4b8.id,
+                             global_num_experts=e)
+        torch.cuda.synchronize()
+        print(f"probe-moe done: 10 calls at T={t}, {int(ti.unique().numel())} experts hit", file=sys.stderr)
         return
     if args.probe_shape:
         name, pm, kind = args.probe_shape.split(":")

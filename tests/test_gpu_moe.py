@@ -196,6 +196,44 @@ def test_moe_gemm_split_k_blocks_of_64(dev):
     assert mtr["max_rel"] <= 2e-2 and mtr["mean_rel"] < 0.04, mtr
 
 
+@pytest.mark.parametrize("m,foreign", [(300, False), (300, True), (1200, False), (8300, False)])
+def test_moe_gemm_tail_tiles_split_on_the_device(dev, m, foreign):
+    """Blocks of 64 with a long K: the 64-row kernel cuts the tiles of its last, partly filled round of resident
+    workgroups along K, by a number of pieces it derives from the live block count on the device, and a second pass adds
+    the pieces.  24 live tiles -> 4 pieces each; 80 -> 4; about 520 -> 512 whole tiles and a few split ones; with blocks
+    of experts held by another rank (left untouched) among them."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    topk, e, bs, k, n = 2, 4, 64, 4096, 1024
+    print(f"tail split m={m} foreign={foreign}", flush=True)
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, 128, torch.float16, False, False, seed=80)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).half()
+    ids = rand_topk(m, topk, e, seed=6)
+    tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7))
+    emap = torch.tensor([0, -1, 1, 2], dtype=torch.int32) if foreign else None
+    local = [0, 2, 3] if foreign else [0, 1, 2, 3]
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e, expert_map=emap.to(dev) if foreign else None)
+    c = torch.full((m * topk, n), 7.0, dtype=torch.float16, device=dev)
+    ws = marlin_make_workspace_new(dev, 4)
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), c, mq[local].to(dev), None, ms[local].to(dev), None, mz[local].to(dev), gi[local].to(dev),
+        perm[local].to(dev), ws, s, x, t, tw.to(dev), moe_block_size=bs, top_k=topk, mul_topk_weights=True, is_ep=foreign,
+        b_q_type=scalar_types.uint4b8, size_m=m, size_n=n, size_k=k, is_k_full=True, use_atomic_add=False,
+        use_fp32_reduce=True, is_zp_float=False).cpu()
+    flat = ids.flatten().long()
+    for ex in range(e):
+        rows = torch.nonzero(flat == ex).flatten()
+        if foreign and ex == 1:
+            assert (out[rows] == 7.0).all()
+            continue
+        ref = (a[rows // topk].float() @ layers[ex].w_ref.float()) * tw.flatten()[rows].unsqueeze(1)
+        mtr = gr.error_metrics(out[rows], ref)
+        assert mtr["max_rel"] <= 2e-2 and mtr["mean_rel"] < 0.04, (ex, mtr)
+    assert int(ws.abs().sum()) == 0
+
+
 def test_moe_gemm_skips_foreign_experts_and_bias(dev):
     """expert_ids = -1 blocks are left untouched (expert parallelism); per-expert bias is added."""
     import vllm_amd.ops as ops

@@ -276,6 +276,10 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       if (sp < 1) sp = 1;
       if (sp > 16) sp = 16;
     }
+    // MoE: the number of live tiles is only known on the device, which then splits K for the tiles of the last, partly
+    // filled round of resident workgroups (two per compute unit); see tail_split
+    const bool tail_dyn = moe && forced_splits <= 0 && pl.total_ksteps >= 3 * TAIL_MIN_KSTEPS;  // (else it never splits)
+    if (tail_dyn) sp = 1;
     if (forced_splits > 0) sp = forced_splits;
     int kps = (int)ceil_div(pl.total_ksteps, sp);
     kps = (kps + 3) / 4 * 4;
@@ -297,9 +301,13 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
       pl.kps = kps;
       pl.xcd_map = 0;
       pl.ctmp_bytes = sp > 1 ? mid_tiles * sp * 64 * 512 * 4 : 0;
+      if (tail_dyn) {
+        pl.dyn_slots = (int)(2 * cus);
+        pl.ctmp_bytes = mid_tail_pieces(mid_tiles, pl.dyn_slots) * 64 * 512 * 4;
+      }
       if (debug_plan)
-        fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=3 tiles=%d splits=%d kps=%d\n", (long long)a->size_m,
-                (long long)a->size_n, (long long)a->size_k, pl.tiles, pl.splits, pl.kps);
+        fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=3 tiles=%d splits=%d kps=%d dyn=%d\n", (long long)a->size_m,
+                (long long)a->size_n, (long long)a->size_k, pl.tiles, pl.splits, pl.kps, pl.dyn_slots);
       return 0;
     }
   }

@@ -30,6 +30,7 @@ struct KParams {
   int xcd_map;
   int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
   int strip0;    // 64-row kernel: first 512-column strip of this launch (it may finish what the prefill kernel left)
+  int dyn_slots; // 64-row kernel, MoE: > 0 = the K split is chosen on the device from the number of live blocks (tail_split)
   // MoE
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
@@ -45,6 +46,35 @@ struct KParams {
   uint32_t* zero_ptr;  // side job: zero_n16 16-byte pieces to clear, spread over the grid
   int64_t zero_n16;
 };
+
+// 64-row kernel on MoE problems.  The number of live tiles L (blocks that hold tokens x column strips) is only known on
+// the device, and whole tiles run in rounds of `slots` resident workgroups.  The tiles of the last, partly filled round
+// (all tiles, when there are fewer than `slots`) are therefore cut along K into S pieces each, as many as still fit that
+// round, and a second pass adds the pieces: F tiles run whole, the R = L - F tail tiles as R * S pieces of kps k-steps
+// (a multiple of 4, at least 32).  Only from S = 3 on: a tail of more than slots / 3 tiles already runs with fewer
+// workgroups per compute unit, hence faster, and halving it gains less than the partial tiles cost.  Both passes derive
+// the same numbers from L.
+constexpr int TAIL_MIN_KSTEPS = 32;
+struct TailSplit {
+  int F, R, S, kps;
+};
+__host__ __device__ inline TailSplit tail_split(int live_tiles, int slots, int total_ksteps) {
+  TailSplit d;
+  d.F = (live_tiles / slots) * slots;
+  d.R = live_tiles - d.F;
+  d.S = 1;
+  d.kps = total_ksteps;
+  if (d.R > 0) {
+    int s = slots / d.R;
+    if (s > 8) s = 8;
+    if (s > total_ksteps / TAIL_MIN_KSTEPS) s = total_ksteps / TAIL_MIN_KSTEPS;
+    if (s >= 3) {
+      d.kps = ((total_ksteps + s - 1) / s + 3) / 4 * 4;
+      d.S = (total_ksteps + d.kps - 1) / d.kps;
+    }
+  }
+  return d;
+}
 
 // Side job of a launch: the grid clears `zero_n16` 16-byte pieces at `zero_ptr` (the output of a later launch that
 // accumulates with atomic adds).  Every workgroup of the grid calls this first, before any early exit.
@@ -189,6 +219,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   p.xcd_map = pl.xcd_map;
   p.tn = pl.tn;
   p.strip0 = pl.strip0;
+  p.dyn_slots = pl.dyn_slots;
   p.sorted_ids = a->sorted_token_ids;
   p.expert_ids = a->expert_ids;
   p.ntpp = a->num_tokens_past_padded;

@@ -54,14 +54,33 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   // tile order: consecutive workgroups walk M first, so workgroups resident together share weight strips
   // (MoE: neighbouring blocks mostly belong to the same expert)
   const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
-  const int mt = blockIdx.x % mtiles;
-  const int split = (blockIdx.x / mtiles) % p.splits, st_l = blockIdx.x / (mtiles * p.splits);
-  const int tile = st_l * mtiles + mt;         // index of the output tile inside this launch (partials)
+  zero_fill_side_job(p);
+  int mt = blockIdx.x % mtiles;
+  int split = (blockIdx.x / mtiles) % p.splits, st_l = blockIdx.x / (mtiles * p.splits);
+  int tile = st_l * mtiles + mt;               // index of the output tile inside this launch (partials)
+  int nsplit = p.splits, kps = p.ksteps_per_split;
+  int moe_ntp = 0;
+  if (MOE) moe_ntp = *p.ntpp;
+  if (MOE && p.dyn_slots > 0) {
+    // live tiles in M-first order; the tail tiles' pieces walk the tiles first, then K (see tail_split)
+    const int live = min((moe_ntp + MD_BM - 1) / MD_BM, mtiles);
+    if (live == 0) return;
+    const TailSplit d = tail_split(live * p.ncp, p.dyn_slots, p.total_ksteps);
+    int j = blockIdx.x;
+    if (j < d.F) {
+      split = 0, nsplit = 1, kps = p.total_ksteps, tile = 0;
+    } else {
+      const int u = j - d.F;
+      if (u >= d.R * d.S) return;
+      tile = u % d.R, split = u / d.R, nsplit = d.S, kps = d.kps;
+      j = d.F + tile;
+    }
+    st_l = j / live, mt = j % live;
+  }
   const int nt4 = p.strip0 + st_l;             // 512-column strip
   const int cp = nt4 * 4 + wv;                 // column pair of this wavefront
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 512: trailing wavefronts only help staging
   const int row0 = mt * MD_BM;
-  zero_fill_side_job(p);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
@@ -69,7 +88,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   const uint16_t* bias = (const uint16_t*)p.bias;
   const uint16_t* gscale = (const uint16_t*)p.gscale;
   if (MOE) {
-    if (row0 >= *p.ntpp) return;
+    if (row0 >= moe_ntp) return;
     const int e = p.expert_ids[mt];
     if (e < 0) return;  // expert of another rank
     Bq += e * p.b_estride;
@@ -129,8 +148,8 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   }
   u32x4 areg[2];
   // this workgroup's k-steps: [ks_b, ks_e), a multiple of 4 long (the host splits K in multiples of 4 k-steps)
-  const int ks_b = split * p.ksteps_per_split;
-  const int ks_e = min(ks_b + p.ksteps_per_split, p.total_ksteps);
+  const int ks_b = split * kps;
+  const int ks_e = min(ks_b + kps, p.total_ksteps);
   // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
   //  keeps the main loop free of branches)
   auto load_a = [&](int chunk) {  // chunk: relative to ks_b
@@ -362,7 +381,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) slab[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
     __builtin_amdgcn_wave_barrier();
-    if (act && p.splits == 1) {
+    if (act && nsplit == 1) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r16 = (lane >> 4) + 4 * i;
@@ -393,11 +412,11 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
       const int r16 = (lane >> 5) + 2 * i;
       const int crow = s_crow[mb * 16 + r16];
       f32x4 v = *(const f32x4*)(slab + r16 * RED_RS + fpos);
-      if (p.splits > 1) {
+      if (nsplit > 1) {
         // K is split: the fp32 partial tile [row 64][column 512] goes to scratch with plain stores; the reduction
         // kernel launched behind this one adds the splits and finishes the rows
         if (fcol_ok && crow >= 0)
-          *(f32x4*)(p.ctmp + (((int64_t)tile * p.splits + split) * MD_BM + mb * 16 + r16) * 512 + wv * 128 + fc4) = v;
+          *(f32x4*)(p.ctmp + (((int64_t)tile * nsplit + split) * MD_BM + mb * 16 + r16) * 512 + wv * 128 + fc4) = v;
         continue;
       }
       if (crow < 0) continue;
@@ -424,7 +443,15 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   const int t = threadIdx.x;
   const int mtiles = MOE ? (p.n_sorted + MD_BM - 1) / MD_BM : (p.M + MD_BM - 1) / MD_BM;
   const int tile = blockIdx.x >> 2, rb = blockIdx.x & 3;
-  const int mt = tile % mtiles, nt4 = p.strip0 + tile / mtiles;
+  int mt = tile % mtiles, nt4 = p.strip0 + tile / mtiles, nsplit = p.splits;
+  if (MOE && p.dyn_slots > 0) {  // tile: index among the tail tiles (see tail_split)
+    const int live = min((*p.ntpp + MD_BM - 1) / MD_BM, mtiles);
+    if (live == 0) return;
+    const TailSplit d = tail_split(live * p.ncp, p.dyn_slots, p.total_ksteps);
+    if (d.S == 1 || tile >= d.R) return;
+    const int j = d.F + tile;
+    mt = j % live, nt4 = p.strip0 + j / live, nsplit = d.S;
+  }
   const int row0 = mt * MD_BM;
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint16_t* bias = (const uint16_t*)p.bias;
@@ -467,7 +494,7 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   };
   col_consts(ncol, cs, bs);
   if (act) col_consts((p.N >> 1) + ncol, cu, bu);
-  const float* parts = p.ctmp + (int64_t)tile * p.splits * (MD_BM * 512) + fc4;
+  const float* parts = p.ctmp + (int64_t)tile * nsplit * (MD_BM * 512) + fc4;
 #pragma unroll 2
   for (int i = 0; i < 8; ++i) {
     const int r = rb * 16 + (t >> 7) + 2 * i;
@@ -480,9 +507,9 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
     }
     if (crow < 0) continue;
     f32x4 v = {0, 0, 0, 0}, u = {0, 0, 0, 0};
-    for (int sidx = 0; sidx < p.splits; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512);
+    for (int sidx = 0; sidx < nsplit; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512);
     if (act)
-      for (int sidx = 0; sidx < p.splits; ++sidx) u += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512 + 64);
+      for (int sidx = 0; sidx < nsplit; ++sidx) u += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512 + 64);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       v[j] = v[j] * cs[j] + bs[j];
@@ -555,8 +582,19 @@ int launch_mid(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
     red = moe ? pick_reduce<DT_BF16, true>(channel) : pick_reduce<DT_BF16, false>(channel);
   }
   KParams p = make_kparams(a, pl);
+  if (pl.tiles <= 0) return 0;
+  if (pl.dyn_slots > 0) {
+    // device-side K split of the tail tiles: at most dyn_slots pieces behind the whole tiles, at most that many tail tiles
+    if (!moe || pl.splits != 1) return fail(W4A16_EINVAL, "unsupported kernel variant");
+    const int64_t pieces = mid_tail_pieces(pl.tiles, pl.dyn_slots);
+    hipLaunchKernelGGL(fn, dim3((unsigned)(pl.tiles + pieces)), dim3(256), MD_SMEM, stream, p);
+    W4A16_HIP(hipGetLastError());
+    const int64_t tail = pl.tiles < pl.dyn_slots ? pl.tiles : pl.dyn_slots;
+    hipLaunchKernelGGL(red, dim3((unsigned)(tail * 4)), dim3(256), 0, stream, p);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
   const int64_t grid = (int64_t)pl.tiles * pl.splits;
-  if (grid <= 0) return 0;
   hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), MD_SMEM, stream, p);
   W4A16_HIP(hipGetLastError());
   if (pl.splits > 1) {

@@ -18,6 +18,7 @@ struct Plan {
   int tn;    // tile width in columns (128; the decode kernel also has 64)
   int nw = 8;  // 16-row tiles (decode kernel, general kernel with one m-block): wavefronts per workgroup (8 or 4)
   int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
+  int dyn_slots = 0;   // 64-row kernel, MoE: resident workgroups that the device-side K split of the tail tiles fills
   int tail_strips = 0; // prefill plan: trailing 512-column strips handed to the 64-row kernel (0 = none)
   int64_t ctmp_bytes;  // fp32 split-K partials
   int64_t atmp_bytes;  // column-permuted copy of A (act-order), after the partials; MoE: one row per sorted slot
@@ -26,6 +27,9 @@ struct Plan {
 // MoE act-order: out[slot, :] = a[sorted_ids[slot] / top_k, perm[expert of the slot's block][:]] for the valid slots
 // (gemm.hip runs it in front of the GEMM kernels, which then read row `slot`).
 int moe_gather_rows(const w4a16_gemm_args* a, void* out, hipStream_t stream);
+
+// 64-row kernel, MoE: upper bound of the tail pieces (tail_split) for a launch of `tiles` tiles at most
+inline int64_t mid_tail_pieces(int64_t tiles, int slots) { return tiles * 8 < slots ? tiles * 8 : slots; }
 
 int launch_skinny(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream);
