@@ -42,15 +42,11 @@ def pick_block_size(tokens: int, topk: int, num_experts: int, expert_bytes: int 
     """Token slots per expert block, from the average expert's share of the slots (the quantity the reference's rule
     uses, fused_marlin_moe.py:279-282), fitted to the kernels behind each size on MI355X: blocks of 16 slots run on the
     weight-streaming kernel, whose cost is one pass over the expert's weights per block; blocks of 64 on the 64-row
-    kernel, which costs about two such passes per block, so it wins once an expert fills more than one and a half
-    blocks of 16 (sooner for experts of a few MB, where the per-block fixed costs count).  Blocks of 32 and 48 only pay
-    while there are too few blocks of 64 to give every compute unit work (few, large experts)."""
+    kernel, which costs about two such passes per block, so it wins once an expert fills more than one and a quarter
+    blocks of 16 (sooner for experts of a few MB, where the per-block fixed costs count).  Blocks of 8 never beat 16,
+    and 32 / 48 lost their niche (few, large experts) when the 64-row kernel began to split K for a thin last round."""
     per_expert = tokens * topk / num_experts
-    if per_expert < (20 if expert_bytes >= (12 << 20) else 14):
-        return 16
-    if num_experts * (per_expert / 64 + 0.5) < 12:
-        return next((bs for bs in (32, 48) if per_expert < 0.9 * bs), 64)
-    return 64
+    return 16 if per_expert < (20 if expert_bytes >= (12 << 20) else 14) else 64
 
 
 @dataclass
