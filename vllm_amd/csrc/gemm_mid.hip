@@ -495,21 +495,39 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   col_consts(ncol, cs, bs);
   if (act) col_consts((p.N >> 1) + ncol, cu, bu);
   const float* parts = p.ctmp + (int64_t)tile * nsplit * (MD_BM * 512) + fc4;
+  // (the rows' slot ids, then per row the partial tiles of four splits at a time, are loaded together: the pass is bound
+  //  by round trips, not by bytes)
+  int crows[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = rb * 16 + (t >> 7) + 2 * i;
+    crows[i] = -1;
+    if (MOE) {
+      const int id = p.sorted_ids[row0 + r];
+      if ((unsigned)id < (unsigned)p.c_rows) crows[i] = id;
+    } else if (row0 + r < p.M) {
+      crows[i] = row0 + r;
+    }
+  }
+  auto sum_splits = [&](const float* src) {  // src: the row's columns in split 0; added in split order
+    f32x4 acc = {0, 0, 0, 0};
+    for (int s0 = 0; s0 < nsplit; s0 += 4) {
+      f32x4 a[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) a[q] = *(const f32x4*)(src + (int64_t)min(s0 + q, nsplit - 1) * (MD_BM * 512));
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (s0 + q < nsplit) acc += a[q];
+    }
+    return acc;
+  };
 #pragma unroll 2
   for (int i = 0; i < 8; ++i) {
     const int r = rb * 16 + (t >> 7) + 2 * i;
-    int crow = -1;
-    if (MOE) {
-      const int id = p.sorted_ids[row0 + r];
-      if ((unsigned)id < (unsigned)p.c_rows) crow = id;
-    } else if (row0 + r < p.M) {
-      crow = row0 + r;
-    }
+    const int crow = crows[i];
     if (crow < 0) continue;
-    f32x4 v = {0, 0, 0, 0}, u = {0, 0, 0, 0};
-    for (int sidx = 0; sidx < nsplit; ++sidx) v += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512);
-    if (act)
-      for (int sidx = 0; sidx < nsplit; ++sidx) u += *(const f32x4*)(parts + ((int64_t)sidx * MD_BM + r) * 512 + 64);
+    f32x4 v = sum_splits(parts + (int64_t)r * 512), u = {0, 0, 0, 0};
+    if (act) u = sum_splits(parts + (int64_t)r * 512 + 64);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       v[j] = v[j] * cs[j] + bs[j];
