@@ -33,7 +33,9 @@ struct DecodeCfg {
   static constexpr int smem(int nw) { return nw * 16 * RS * 4; }
 };
 
-template <int DT, bool ZP, bool CHANNEL, int TN, int DNW>
+// MOE: the launch walks MoE blocks (slot ids, expert ids, fused epilogues); the dense instantiations carry none of that
+// code, which shortens the chain of argument loads in front of a small layer's first weight load
+template <int DT, bool ZP, bool CHANNEL, int TN, int DNW, bool MOE>
 __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   constexpr int W = TN / 32;  // Marlin words per lane and k-tile: 4 (128-bit load) or 2 (64-bit load)
   constexpr bool HI_TRICK = (DT == DT_F16) && !ZP;
@@ -48,20 +50,27 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   // weight-side roles: c = column inside an 8-column block, h = which half of the tile's columns, g = K group
   const int c = lane & 7, h = (lane >> 3) & 1, g = lane >> 4;
 
+  // The grid is three-dimensional so that (tile, split) come from the block indices without an integer division (a
+  // small layer's first weight load waits for every instruction in front of it); workgroups are dispatched x fastest:
+  //   plain:   x = split, y + 65535 z = tile                       (the splits of a tile are neighbours)
+  //   xcd_map: x = tile % 8, y = split, z = tile / 8               (consecutive workgroups go round the eight XCDs, so
+  //            all splits of a tile share one XCD's L2)
   int tile, split;
-  {
-    const int b = blockIdx.x;
-    if (p.xcd_map) {
-      const int idx = b >> 3;
-      tile = (idx / p.splits) * 8 + (b & 7);
-      split = idx % p.splits;
-    } else {
-      tile = b / p.splits;
-      split = b % p.splits;
-    }
+  if (p.xcd_map) {
+    tile = blockIdx.z * 8 + blockIdx.x;
+    split = blockIdx.y;
+  } else {
+    tile = blockIdx.z * 65535 + blockIdx.y;
+    split = blockIdx.x;
+    if (tile >= p.tiles) return;
   }
-  const int ct = tile % p.ncp, mt = tile / p.ncp;  // column tile, m-tile
-  zero_fill_side_job(p);
+  int ct = tile, mt = 0;  // column tile, m-tile
+  if (p.ncp != p.tiles) {
+    ct = tile % p.ncp;
+    mt = tile / p.ncp;
+  }
+  if constexpr (MOE)
+    zero_fill_side_job(p, (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x, gridDim.x * gridDim.y * gridDim.z);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
@@ -75,7 +84,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   // block's expert and the number of live slots, all loaded together: a workgroup then waits for one round trip, not
   // five in a row, before it can address its weights and activations (short-K expert GEMMs live only a few of them)
   int id_0 = 0, id_a0 = 0, id_a1 = 0, id_t = 0, moe_e = 0, moe_ntp = 0;
-  if (p.moe) {
+  if constexpr (MOE) {
     const int* ids = p.sorted_ids + mt * p.moe_bs;
     const int last = p.moe_bs - 1;
     id_0 = ids[0];
@@ -89,7 +98,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   auto tile_row_ids = [&](int r, int id, int& src, int& dst) {
     src = -1;
     dst = -1;
-    if (p.moe) {
+    if constexpr (MOE) {
       if (r < p.moe_bs && (unsigned)id < (unsigned)p.c_rows) {
         src = p.a_by_slot ? mt * p.moe_bs + r : id / p.top_k;
         dst = id;
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     tile_row_ids(tr, id_t, src, dst);
     s_crow[tr] = dst;
   }
-  if (p.moe) {
+  if constexpr (MOE) {
     if (mt * p.moe_bs >= moe_ntp || moe_e < 0) return;
     Bq += moe_e * p.b_estride;
     Sc += moe_e * p.s_estride;
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   // n-tile this lane reads (TN=128: 2ct+h, TN=64: ct); a missing second n-tile (N/64 odd) aliases n-tile 0
   int nt;
   if (TN == 128)  // (fused SiLU-and-mul: gate n-tile ct paired with the up n-tile of the same output columns)
-    nt = p.act ? (h ? (p.N >> 7) + ct : ct) : ((2 * ct + h) * 64 < p.N ? 2 * ct + h : 0);
+    nt = (MOE && p.act) ? (h ? (p.N >> 7) + ct : ct) : ((2 * ct + h) * 64 < p.N ? 2 * ct + h : 0);
   else
     nt = ct;
   const int64_t b_row = (int64_t)p.N * 2;  // words per k-tile row
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
 
   // rows 8..15 of the tile exist?  (otherwise their activation loads are skipped)
-  const bool rows_hi = p.moe ? (p.moe_bs > 8) : (mt * 16 + 8 < p.M);
+  const bool rows_hi = MOE ? (p.moe_bs > 8) : (mt * 16 + 8 < p.M);
   // scale group of an absolute stage index (channel-wise scales: pseudo-groups of 128 K rows, so that the raw partial
   // sums, biased by E * sum(a), stay small next to fp32's 24 bits whatever the activations' mean)
   auto group_of = [&](int sidx) {
@@ -345,19 +354,19 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
         v[j] += (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
       }
     }
-    if (p.mul_topk) {
+    if (MOE && p.mul_topk) {
       const float tw = p.topk_w[crow];
 #pragma unroll
       for (int j = 0; j < CPT; ++j) v[j] *= tw;
     }
   };
   // fused SiLU-and-mul (TN = 128 only, host-checked): the threads of the gate half also take the up half's columns
-  const bool act_lane = TN == 128 && p.act && fc < 64;
+  const bool act_lane = MOE && TN == 128 && p.act && fc < 64;
   auto finalize = [&](float* v, float* u, int fr) {
     const int crow = s_crow[fr];
     if (crow < 0) return;
     if constexpr (TN == 128) {
-      if (p.act) {
+      if (MOE && p.act) {
         if (!act_lane) return;
         const int oc = ct * 64 + fc;
         finish(v, oc, crow);
@@ -372,7 +381,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
       store_row4<DT>(p, crow, ncol, f32x4{v[0], v[1], v[2], v[3]});
     } else {
       const uint32_t o = pack2<DT>(v[0], v[1]);
-      if (p.sum_div > 0) {
+      if (MOE && p.sum_div > 0) {
         uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * p.N + ncol;
         if constexpr (DT == DT_F16) {
           typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -476,36 +485,48 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
 // ------------------------------------------------------------------------------------ host side
 typedef void (*decode_fn)(const KParams);
 
+template <int DT, int TN, int NW, bool MOE>
+static decode_fn pick5(bool zp, bool channel) {
+  if (zp) return channel ? decode_kernel<DT, true, true, TN, NW, MOE> : decode_kernel<DT, true, false, TN, NW, MOE>;
+  return channel ? decode_kernel<DT, false, true, TN, NW, MOE> : decode_kernel<DT, false, false, TN, NW, MOE>;
+}
 template <int DT, int TN, int NW>
-static decode_fn pick4(bool zp, bool channel) {
-  if (zp) return channel ? decode_kernel<DT, true, true, TN, NW> : decode_kernel<DT, true, false, TN, NW>;
-  return channel ? decode_kernel<DT, false, true, TN, NW> : decode_kernel<DT, false, false, TN, NW>;
+static decode_fn pick4(bool moe, bool zp, bool channel) {
+  return moe ? pick5<DT, TN, NW, true>(zp, channel) : pick5<DT, TN, NW, false>(zp, channel);
 }
 template <int DT, int TN>
-static decode_fn pick3(int nw, bool zp, bool channel) {
-  return nw == 4 ? pick4<DT, TN, 4>(zp, channel) : pick4<DT, TN, 8>(zp, channel);
+static decode_fn pick3(int nw, bool moe, bool zp, bool channel) {
+  return nw == 4 ? pick4<DT, TN, 4>(moe, zp, channel) : pick4<DT, TN, 8>(moe, zp, channel);
 }
 template <int DT>
-static decode_fn pick2(int tn, int nw, bool zp, bool channel) {
-  return tn == 64 ? pick3<DT, 64>(nw, zp, channel) : pick3<DT, 128>(nw, zp, channel);
+static decode_fn pick2(int tn, int nw, bool moe, bool zp, bool channel) {
+  return tn == 64 ? pick3<DT, 64>(nw, moe, zp, channel) : pick3<DT, 128>(nw, moe, zp, channel);
 }
 
 // (act-order never reaches the kernel as such: the host gathers A's columns in front of the launch, see gemm.hip)
-static decode_fn pick_decode(int dt, int tn, int nw, bool zp, bool channel) {
-  return dt == DT_F16 ? pick2<DT_F16>(tn, nw, zp, channel) : pick2<DT_BF16>(tn, nw, zp, channel);
+static decode_fn pick_decode(int dt, int tn, int nw, bool moe, bool zp, bool channel) {
+  return dt == DT_F16 ? pick2<DT_F16>(tn, nw, moe, zp, channel) : pick2<DT_BF16>(tn, nw, moe, zp, channel);
 }
 
 int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr;
   if (pl.use_perm) return fail(W4A16_EINVAL, "unsupported kernel variant");
   const int nw = pl.nw == 4 ? 4 : 8;
-  decode_fn fn = pick_decode(a->dtype, pl.tn, nw, zp, pl.gm == GM_CHANNEL);
+  decode_fn fn = pick_decode(a->dtype, pl.tn, nw, (a->flags & W4A16_F_MOE) != 0, zp, pl.gm == GM_CHANNEL);
   KParams p = make_kparams(a, pl);
   const int smem = pl.tn == 64 ? DecodeCfg<64>::smem(nw) : DecodeCfg<128>::smem(nw);
   W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
-  const int64_t grid = (int64_t)pl.tiles * pl.splits;
-  if (grid <= 0) return 0;
-  hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(nw * 64), smem, stream, p);
+  if ((int64_t)pl.tiles * pl.splits <= 0) return 0;
+  dim3 grid;
+  if (pl.xcd_map) {
+    if (pl.tiles % 8 != 0 || pl.tiles / 8 > 65535 || pl.splits > 65535) return fail(W4A16_EINVAL, "unsupported launch shape");
+    grid = dim3(8, (unsigned)pl.splits, (unsigned)(pl.tiles / 8));
+  } else {
+    if (pl.splits > 65535) return fail(W4A16_EINVAL, "unsupported launch shape");
+    const unsigned gy = pl.tiles < 65535 ? (unsigned)pl.tiles : 65535u;
+    grid = dim3((unsigned)pl.splits, gy, (unsigned)((pl.tiles + 65534) / 65535));
+  }
+  hipLaunchKernelGGL(fn, grid, dim3(nw * 64), smem, stream, p);
   W4A16_HIP(hipGetLastError());
   return 0;
 }

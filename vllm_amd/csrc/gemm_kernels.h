@@ -25,7 +25,8 @@ struct KParams {
   int N, K;
   int group_ksteps;  // GM_GROUPED: group_size / 32
   int group_shift;   // log2(group_ksteps) when that is a power of two, else -1
-  int ncp;           // column pairs = ceil(N / 128)
+  int ncp;           // column tiles = ceil(N / tile width)
+  int tiles;         // output tiles of the launch (ncp x m-tiles)
   int splits, ksteps_per_split, total_ksteps;
   int xcd_map;
   int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
@@ -78,12 +79,13 @@ __host__ __device__ inline TailSplit tail_split(int live_tiles, int slots, int t
 
 // Side job of a launch: the grid clears `zero_n16` 16-byte pieces at `zero_ptr` (the output of a later launch that
 // accumulates with atomic adds).  Every workgroup of the grid calls this first, before any early exit.
-__device__ __forceinline__ void zero_fill_side_job(const KParams& p) {
+__device__ __forceinline__ void zero_fill_side_job(const KParams& p, unsigned block, unsigned nblocks) {
   if (p.zero_n16 <= 0) return;
-  const int64_t per = (p.zero_n16 + gridDim.x - 1) / gridDim.x;
-  const int64_t b = (int64_t)blockIdx.x * per, e = b + per < p.zero_n16 ? b + per : p.zero_n16;
+  const int64_t per = (p.zero_n16 + nblocks - 1) / nblocks;
+  const int64_t b = (int64_t)block * per, e = b + per < p.zero_n16 ? b + per : p.zero_n16;
   for (int64_t i = b + threadIdx.x; i < e; i += blockDim.x) ((u32x4*)p.zero_ptr)[i] = u32x4{0, 0, 0, 0};
 }
+__device__ __forceinline__ void zero_fill_side_job(const KParams& p) { zero_fill_side_job(p, blockIdx.x, gridDim.x); }
 
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -213,6 +215,7 @@ inline KParams make_kparams(const w4a16_gemm_args* a, const Plan& pl) {
   for (int sh = 0; sh < 20; ++sh)
     if ((1 << sh) == pl.group_ksteps) p.group_shift = sh;
   p.ncp = pl.ncp;
+  p.tiles = pl.tiles;
   p.splits = pl.splits;
   p.ksteps_per_split = pl.kps;
   p.total_ksteps = pl.total_ksteps;
