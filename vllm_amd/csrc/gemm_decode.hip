@@ -378,7 +378,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     if (!fcol_ok) return;
     finish(v, ncol, crow);
     if constexpr (CPT == 4) {
-      store_row4<DT>(p, crow, ncol, f32x4{v[0], v[1], v[2], v[3]});
+      store_row4<DT, MOE>(p, crow, ncol, f32x4{v[0], v[1], v[2], v[3]});
     } else {
       const uint32_t o = pack2<DT>(v[0], v[1]);
       if (MOE && p.sum_div > 0) {

@@ -98,10 +98,10 @@ __device__ __forceinline__ float hi_f32(uint32_t x) { return DT == DT_F16 ? f16_
 
 // Four finished fp32 results of C row `crow`, columns ncol .. ncol + 3: rounded to the 16-bit type, then stored, or
 // (sum_div > 0) added into row crow / sum_div with packed 16-bit atomic adds.
-template <int DT>
+template <int DT, bool MOE = true>
 __device__ __forceinline__ void store_row4(const KParams& p, int crow, int ncol, f32x4 v) {
   const uint32_t o0 = pack2<DT>(v[0], v[1]), o1 = pack2<DT>(v[2], v[3]);
-  if (p.sum_div > 0) {
+  if (MOE && p.sum_div > 0) {
     uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * p.N + ncol;
     if constexpr (DT == DT_F16) {
       typedef _Float16 h2 __attribute__((ext_vector_type(2)));
