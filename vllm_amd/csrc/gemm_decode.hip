@@ -43,6 +43,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   using bvec = uint32_t __attribute__((ext_vector_type(W)));
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[16];
+  __shared__ float s_tw[16];  // MoE: routing weight of each tile row
   __shared__ int s_last;
 
   const int lane = threadIdx.x & 63;
@@ -124,6 +125,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     int src, dst;
     tile_row_ids(tr, id_t, src, dst);
     s_crow[tr] = dst;
+    if (MOE && p.mul_topk) s_tw[tr] = dst >= 0 ? p.topk_w[dst] : 0.f;
   }
   if constexpr (MOE) {
     if (mt * p.moe_bs >= moe_ntp || moe_e < 0) return;
@@ -337,31 +339,53 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   const bool single = p.splits == 1;
   float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (16 * TN);
 
-  // channel scale, bias and routing weight of CPT finished columns starting at real column `col`
-  auto finish = [&](float* v, int col, int crow) {
+  // channel scale and bias of CPT finished columns starting at real column `col`; read once, in front of the barriers
+  // below (inside the row passes every load would wait behind the stores of the pass before)
+  auto col_consts = [&](int col, float* sc, float* bo) {
     const int base = col & ~31, cl = col & 31;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      sc[j] = 1.0f;
+      bo[j] = 0.0f;
+      if (CHANNEL) {
+        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
+        sc[j] = (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
+      }
+      if (bias) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        bo[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+  };
+  // ... applied, with the row's routing weight, to finished values
+  auto finish = [&](float* v, const float* sc, const float* bo, int fr) {
     if (CHANNEL) {
 #pragma unroll
-      for (int j = 0; j < CPT; ++j) {
-        const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        v[j] *= (DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv);
-      }
+      for (int j = 0; j < CPT; ++j) v[j] *= sc[j];
     }
     if (bias) {
 #pragma unroll
-      for (int j = 0; j < CPT; ++j) {
-        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
-        v[j] += (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
-      }
+      for (int j = 0; j < CPT; ++j) v[j] += bo[j];
     }
     if (MOE && p.mul_topk) {
-      const float tw = p.topk_w[crow];
+      const float tw = s_tw[fr];
 #pragma unroll
       for (int j = 0; j < CPT; ++j) v[j] *= tw;
     }
   };
   // fused SiLU-and-mul (TN = 128 only, host-checked): the threads of the gate half also take the up half's columns
   const bool act_lane = MOE && TN == 128 && p.act && fc < 64;
+  float cs[CPT], bs[CPT], cu[CPT], bu[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) cs[j] = cu[j] = 1.0f, bs[j] = bu[j] = 0.0f;
+  if (MOE && TN == 128 && p.act) {
+    if (act_lane) {
+      col_consts(ct * 64 + fc, cs, bs);
+      col_consts((p.N >> 1) + ct * 64 + fc, cu, bu);
+    }
+  } else if (fcol_ok) {
+    col_consts(ncol, cs, bs);
+  }
   auto finalize = [&](float* v, float* u, int fr) {
     const int crow = s_crow[fr];
     if (crow < 0) return;
@@ -369,14 +393,14 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
       if (MOE && p.act) {
         if (!act_lane) return;
         const int oc = ct * 64 + fc;
-        finish(v, oc, crow);
-        finish(u, (p.N >> 1) + oc, crow);
+        finish(v, cs, bs, fr);
+        finish(u, cu, bu, fr);
         store_row4_silu_mul<DT>(p, crow, oc, f32x4{v[0], v[1], v[2], v[3]}, f32x4{u[0], u[1], u[2], u[3]});
         return;
       }
     }
     if (!fcol_ok) return;
-    finish(v, ncol, crow);
+    finish(v, cs, bs, fr);
     if constexpr (CPT == 4) {
       store_row4<DT, MOE>(p, crow, ncol, f32x4{v[0], v[1], v[2], v[3]});
     } else {

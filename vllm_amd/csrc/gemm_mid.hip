@@ -30,7 +30,7 @@ constexpr int MD_BM = 64;    // rows per tile
 constexpr int MD_D = 4;      // weight k-steps in flight per wavefront
 constexpr int MD_ABUF = 2 * MD_MB * 64 * 16;            // one A buffer: 2 k-steps x 4 m-blocks x 64 lanes x 16 B
 constexpr int MD_SLABS = 4 * 16 * RED_RS * 4;           // four wavefront slabs of the epilogue
-constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_BM * 4;  // + C row of each tile row
+constexpr int MD_SMEM = (2 * MD_ABUF > MD_SLABS ? 2 * MD_ABUF : MD_SLABS) + MD_BM * 8;  // + C row and routing weight of each tile row
 
 // FP4 = 1 / 2: float4_e2m1f weights with NVFP4 / MXFP4 scale records (one 16-byte record per lane and k-step / two
 // k-steps); NVFP4's per-expert global scale is applied to the accumulator.
@@ -45,7 +45,8 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
   static_assert(!FP8 || BITS == 8, "fp8 weights use the 8-bit layout");
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
-  int* s_crow = (int*)(smem + MD_SMEM - MD_BM * 4);
+  int* s_crow = (int*)(smem + MD_SMEM - MD_BM * 8);
+  float* s_tw = (float*)(smem + MD_SMEM - MD_BM * 4);
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wv = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -114,6 +115,8 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
     int src, dst;
     tile_row_ids(t, src, dst);
     s_crow[t] = dst;
+    // (read here once: in the epilogue a load per row would wait behind every store in front of it)
+    if (MOE && p.mul_topk) s_tw[t] = dst >= 0 ? p.topk_w[dst] : 0.f;
   }
 
   // ---- weights of this wavefront
@@ -395,7 +398,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
           u[j] = u[j] * cu[j] + bu[j];
         }
         if (p.mul_topk) {
-          const float tw = p.topk_w[crow];
+          const float tw = s_tw[mb * 16 + r16];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             v[j] *= tw;
@@ -424,7 +427,7 @@ __global__ __launch_bounds__(256, 2) void mid_kernel(const KParams p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = v[j] * cs[j] + bs[j];
         if (MOE && p.mul_topk) {
-          const float tw = p.topk_w[crow];
+          const float tw = s_tw[mb * 16 + r16];
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] *= tw;
         }
@@ -498,6 +501,7 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
   // (the rows' slot ids, then per row the partial tiles of four splits at a time, are loaded together: the pass is bound
   //  by round trips, not by bytes)
   int crows[8];
+  float tws[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int r = rb * 16 + (t >> 7) + 2 * i;
@@ -509,6 +513,8 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
       crows[i] = row0 + r;
     }
   }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) tws[i] = (MOE && p.mul_topk && crows[i] >= 0) ? p.topk_w[crows[i]] : 1.0f;
   auto sum_splits = [&](const float* src) {  // src: the row's columns in split 0; added in split order
     f32x4 acc = {0, 0, 0, 0};
     for (int s0 = 0; s0 < nsplit; s0 += 4) {
@@ -534,7 +540,7 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const KParams p) {
       u[j] = u[j] * cu[j] + bu[j];
     }
     if (MOE && p.mul_topk) {
-      const float tw = p.topk_w[crow];
+      const float tw = tws[i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         v[j] *= tw;

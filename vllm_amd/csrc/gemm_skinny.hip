@@ -67,6 +67,7 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
   constexpr bool A_PAIR_ORDER = FP4_DIRECT || FP8_DIRECT;  // A fragments in the K order (k0, k0+8, k0+1, k0+9, ...)
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int s_crow[BM];  // C row of each tile row, -1 = not written
+  __shared__ float s_tw[BM];  // MoE: routing weight of each tile row
   __shared__ int s_last;
 
   const int lane = threadIdx.x & 63;
@@ -146,6 +147,7 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
     int src, dst;
     tile_row_ids(tr, id_t, src, dst);
     s_crow[tr] = dst;
+    if (p.mul_topk) s_tw[tr] = dst >= 0 ? p.topk_w[dst] : 0.f;
   }
   if (p.moe) {
     if (mt * p.moe_bs >= moe_ntp || moe_e < 0) return;
@@ -478,33 +480,50 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
   const bool single = p.splits == 1;
   float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (BM * 128);
 
-  // channel scale, global scale, bias and routing weight of four finished columns starting at real column `col`
-  auto finish = [&](f32x4 v, int col, int crow) {
+  // channel scale (times the global scale) and bias of four finished columns starting at real column `col`; read once,
+  // in front of the m-block loop (inside it every load would wait behind the stores of the rows before)
+  struct ColConsts { f32x4 sc, bo; };
+  auto col_consts = [&](int col) {
+    ColConsts cc{f32x4{1.f, 1.f, 1.f, 1.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    const int base = col & ~31, cl = col & 31;
     if (GM == GM_CHANNEL) {
-      const int base = col & ~31, cl = col & 31;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint16_t sv = Sc[base + single_perm_pos(cl + j)];
-        v[j] *= ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (FP8 ? fp8_scale_unbias<DT>() : 1.0f);
+        cc.sc[j] = ((DT == DT_F16) ? f16_lo_f32(sv) : bf16_lo_f32(sv)) * (FP8 ? fp8_scale_unbias<DT>() : 1.0f);
       }
     }
+    if (bias) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
+        cc.bo[j] = (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
+      }
+    }
+    return cc;
+  };
+  float gs = 1.0f;
+  if constexpr (FP4 == 1) {
+    // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
+    const uint16_t gv = *gscale;
+    gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
+  }
+  // ... applied, with the row's routing weight, to finished values
+  auto finish = [&](f32x4 v, const ColConsts& cc, int r) {
+    if (GM == GM_CHANNEL) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] *= cc.sc[j];
+    }
     if constexpr (FP4 == 1) {
-      // NVFP4 global scale: stored times 2^7 (fp16) / 2^119 (bf16) by the reference's load-time processing
-      const uint16_t gv = *gscale;
-      const float gs = (DT == DT_F16) ? f16_lo_f32(gv) * 0x1.0p-7f : bf16_lo_f32(gv) * 0x1.0p-119f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] *= gs;
     }
     if (bias) {
-      const int base = col & ~31, cl = col & 31;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint16_t bv = bias[base + single_perm_pos(cl + j)];
-        v[j] += (DT == DT_F16) ? f16_lo_f32(bv) : bf16_lo_f32(bv);
-      }
+      for (int j = 0; j < 4; ++j) v[j] += cc.bo[j];
     }
     if (p.mul_topk) {
-      const float tw = p.topk_w[crow];
+      const float tw = s_tw[r];
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] *= tw;
     }
@@ -512,15 +531,23 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
   };
   // v: the thread's four columns; u (fused SiLU-and-mul, threads of the gate half only): the up half's same columns
   const bool act_lane = p.act && fc4 < 64;
+  ColConsts ccv{f32x4{1.f, 1.f, 1.f, 1.f}, f32x4{0.f, 0.f, 0.f, 0.f}}, ccu = ccv;
+  if (p.act) {
+    if (act_lane) {
+      ccv = col_consts(cp * 64 + fc4);
+      ccu = col_consts((p.N >> 1) + cp * 64 + fc4);
+    }
+  } else if (fcol_ok) {
+    ccv = col_consts(ncol);
+  }
   auto finalize = [&](int r, f32x4 v, f32x4 u) {
     const int crow = s_crow[r];
     if (crow < 0) return;
     if (p.act) {
       if (!act_lane) return;
-      const int oc = cp * 64 + fc4;
-      store_row4_silu_mul<DT>(p, crow, oc, finish(v, oc, crow), finish(u, (p.N >> 1) + oc, crow));
+      store_row4_silu_mul<DT>(p, crow, cp * 64 + fc4, finish(v, ccv, r), finish(u, ccu, r));
     } else if (fcol_ok) {
-      store_row4<DT>(p, crow, ncol, finish(v, ncol, crow));
+      store_row4<DT>(p, crow, ncol, finish(v, ccv, r));
     }
   };
 
