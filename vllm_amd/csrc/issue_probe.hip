@@ -49,7 +49,68 @@ __global__ __launch_bounds__(512) void issue_probe_kernel(const uint32_t* __rest
   out[(size_t)blockIdx.x * blockDim.x + t] = s + (float)x;
 }
 
+// The same loop on v_mfma_f32_32x32x16_f16: 8 independent accumulators of 16 registers, 32768 flop per MFMA, so that
+// NV VALU instructions per MFMA here are the same VALU work per flop as NV / 2 above.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+template <int NV, bool DEP>
+__global__ __launch_bounds__(512) void issue_probe32_kernel(const uint32_t* __restrict__ in, float* __restrict__ out, int iters) {
+  f32x16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.0f;
+  const int t = threadIdx.x;
+  u32x4 a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = *(const u32x4*)(in + ((t * 6 + i) * 4) % 4096);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) b[i] = *(const u32x4*)(in + ((t * 6 + 4 + i) * 4) % 4096);
+  uint32_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = in[(t + 11 * i) % 4096];
+  uint32_t mask = 0x000f000fu, ex = 0x64006400u;
+  asm volatile("" : "+v"(mask), "+v"(ex));
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a[i >> 1]), "v"(b[i & 1]));
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+          if (DEP)
+            asm volatile("v_and_or_b32 %0, %0, %1, %2" : "+v"(v[0]) : "v"(mask), "v"(ex));
+          else
+            asm volatile("v_and_or_b32 %0, %0, %1, %2" : "+v"(v[(i * NV + j) & 7]) : "v"(mask), "v"(ex));
+        }
+      }
+    }
+  }
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  float s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  uint32_t x = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x ^= v[i];
+  out[(size_t)blockIdx.x * blockDim.x + t] = s + (float)x;
+}
+
 typedef void (*probe_fn)(const uint32_t*, float*, int);
+template <bool DEP>
+static probe_fn pick32(int nv) {
+  switch (nv) {
+    case 0: return issue_probe32_kernel<0, DEP>;
+    case 2: return issue_probe32_kernel<2, DEP>;
+    case 4: return issue_probe32_kernel<4, DEP>;
+    case 6: return issue_probe32_kernel<6, DEP>;
+    case 8: return issue_probe32_kernel<8, DEP>;
+    case 12: return issue_probe32_kernel<12, DEP>;
+    default: return nullptr;
+  }
+}
 template <bool DEP>
 static probe_fn pick(int nv) {
   switch (nv) {
@@ -65,10 +126,11 @@ static probe_fn pick(int nv) {
 }
 
 // in: 4096 dwords of operand data on the device; out: >= workgroups * 512 floats.  Returns the best of three timed
-// launches in milliseconds (negative on error).  MFMAs per wavefront = iters * 32.
+// launches in milliseconds (negative on error).  MFMAs per wavefront = iters * 32 (shape 0: 16x16x32) or iters * 16
+// (shape 1: 32x32x16), the same flops.
 extern "C" float w4a16_issue_probe(const uint32_t* in, float* out, int workgroups, int waves_per_wg, int nv, int dependent,
-                                   int iters) {
-  probe_fn fn = dependent ? pick<true>(nv) : pick<false>(nv);
+                                   int iters, int shape) {
+  probe_fn fn = shape == 1 ? (dependent ? pick32<true>(nv) : pick32<false>(nv)) : (dependent ? pick<true>(nv) : pick<false>(nv));
   if (!fn || (waves_per_wg != 4 && waves_per_wg != 8) || workgroups <= 0) return -1.0f;
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -2.0f;

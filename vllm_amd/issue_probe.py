@@ -16,7 +16,7 @@ def run(dev, iters: int = 2000) -> list[dict]:
     lib = ctypes.CDLL(LIB_PATH)
     lib.w4a16_issue_probe.restype = ctypes.c_float
     lib.w4a16_issue_probe.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                      ctypes.c_int, ctypes.c_int]
+                                      ctypes.c_int, ctypes.c_int, ctypes.c_int]
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     g = torch.Generator().manual_seed(1)
     rnd = (torch.rand(8192, generator=g) * 4 - 2).half().view(torch.int32).to(dev)       # 4096 dwords of fp16 pairs
@@ -32,7 +32,7 @@ def run(dev, iters: int = 2000) -> list[dict]:
                         continue
                     if data == "zeros" and (nv > 0):
                         continue
-                    ms = lib.w4a16_issue_probe(src.data_ptr(), out.data_ptr(), cus, waves, nv, dep, iters)
+                    ms = lib.w4a16_issue_probe(src.data_ptr(), out.data_ptr(), cus, waves, nv, dep, iters, 0)
                     assert ms > 0, ms
                     per_simd_ns = ms * 1e6 / (iters * 32 * waves / 4)
                     tflops = cus * waves * iters * 32 * 16384.0 / (ms * 1e-3) / 1e12
@@ -40,6 +40,16 @@ def run(dev, iters: int = 2000) -> list[dict]:
                                      ns_per_mfma_per_simd=per_simd_ns, tflops=tflops))
                     print(f"{data:6s} waves/SIMD={waves // 4} VALU/MFMA={nv} {'chained' if dep else 'independent'}: "
                           f"{per_simd_ns:6.2f} ns per MFMA and SIMD, {tflops:7.0f} TFLOP/s", flush=True)
+    # the same VALU work per flop on v_mfma_f32_32x32x16_f16 (half as many, twice as long MFMAs)
+    for waves in (4, 8):
+        for nv in (0, 2, 4, 6, 8, 12):
+            ms = lib.w4a16_issue_probe(rnd.data_ptr(), out.data_ptr(), cus, waves, nv, 0, iters, 1)
+            assert ms > 0, ms
+            tflops = cus * waves * iters * 16 * 32768.0 / (ms * 1e-3) / 1e12
+            rows.append(dict(data="random", mfma="32x32x16", waves_per_simd=waves // 4, valu_per_mfma=nv, dependent=False,
+                             ns_per_mfma_per_simd=ms * 1e6 / (iters * 16 * waves / 4), tflops=tflops))
+            print(f"random 32x32x16 waves/SIMD={waves // 4} VALU/MFMA={nv} (= {nv / 2:g} per 16384 flop) independent: "
+                  f"{tflops:7.0f} TFLOP/s", flush=True)
     return rows
 
 
