@@ -279,6 +279,39 @@ def bench_moe(ops, wtype, dev):
     return out
 
 
+def bench_moe_fine_grained(dev):
+    """A fine-grained MoE layer (128 experts, hidden 2048, intermediate 768, top-8: the shape of Qwen3-30B-A3B), uint4b8
+    g128 fp16 with random codes and scales, T in {16, 512, 4096}; one call = fused_marlin_moe (parity is the tests'
+    business; this row only times the launch sequence)."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    from vllm_amd.scalar_type import scalar_types
+    e, hid, inter, topk = 128, 2048, 768, 8
+    gen = torch.Generator(device=dev).manual_seed(3)
+    codes = lambda *shape: torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device=dev, generator=gen)
+    scales = lambda *shape: (torch.rand(shape, device=dev, generator=gen) * 0.01 + 0.001).half()
+    q1, s1 = codes(e, hid // 16, 2 * inter * 2), scales(e, hid // GROUP, 2 * inter)
+    q2, s2 = codes(e, inter // 16, hid * 2), scales(e, inter // GROUP, hid)
+    per_expert = (hid * 2 * inter + inter * hid) // 2 + ((hid // GROUP) * 2 * inter + (inter // GROUP) * hid) * 2
+    out = {}
+    for t in (16, 512, 4096):
+        x = (torch.randn(t, hid, device=dev, generator=gen) / 10).half()
+        logits = torch.randn(t, e, device=dev, generator=gen)
+        tw, ti = torch.topk(torch.softmax(logits, dim=-1), topk)
+        tw, ti = (tw / tw.sum(dim=-1, keepdim=True)).contiguous(), ti.to(torch.int32).contiguous()
+        call = lambda: fused_marlin_moe(x, q1, q2, None, None, s1, s2, logits, tw, ti,
+                                        quant_type_id=scalar_types.uint4b8.id, global_num_experts=e)
+        call()
+        sec = time_graph([call] * 4, reps=3, warmup=1) / 4
+        hit = int(ti.unique().numel())
+        by = hit * per_expert + t * hid * 2 * 2 + t * topk * (2 * inter + inter + hid) * 2 * 2
+        fl = 2.0 * t * topk * (hid * 2 * inter + inter * hid)
+        out[f"T{t}"] = {"tokens": t, "experts_hit": hit, "us": sec * 1e6, "GBps": by / sec / 1e9, "TFLOPs": fl / sec / 1e12,
+                        "hbm_frac": by / sec / 1e9 / HBM_PEAK_GBPS, "mfma_frac": fl / sec / 1e12 / MFMA_PEAK_TFLOPS}
+        print(f"[detail] 128-expert top-8 moe T={t}: {sec * 1e6:.1f} us, {by / sec / 1e9:.0f} GB/s = "
+              f"{100 * by / sec / 1e9 / HBM_PEAK_GBPS:.1f}% HBM, {fl / sec / 1e12:.1f} TFLOP/s", file=sys.stderr, flush=True)
+    return out
+
+
 def bench_other_types(ops, dev, workspace):
     """The other weight types of the operator on gate_up (4096 x 28672): uint8b128, float8_e4m3fn, NVFP4, MXFP4 and
     uint4 with fp16 zero points, at M = 16 and M = 4096 (warm weights, random codes; parity is the tests' business)."""
@@ -559,7 +592,7 @@ def main():
     if not args.no_detail:
         detail = {"decode_fp16_gptq": {}, "prefill_bf16_awq": {}}  # + act_order_fp16_gptq, mixtral_moe_fp16_gptq
         for name, (k, n) in LAYERS.items():
-            for mm in (1, 4, 16, 64, 256):
+            for mm in (1, 4, 16, 64, 256, 1024):
                 r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_layer(ops, *a), mm, k, n,
                                 torch.float16, dev, workspace)
                 detail["decode_fp16_gptq"][f"{name}_M{mm}"] = r
@@ -575,6 +608,8 @@ def main():
         detail["act_order_fp16_gptq"] = bench_act_order(ops, scalar_types.uint4b8, dev, workspace)
         torch.cuda.empty_cache()
         detail["mixtral_moe_fp16_gptq"] = bench_moe(ops, scalar_types.uint4b8, dev)
+        torch.cuda.empty_cache()
+        detail["fine_grained_moe_fp16_gptq"] = bench_moe_fine_grained(dev)
         torch.cuda.empty_cache()
         detail["repack"] = bench_repack(ops, dev)
         detail["load_path"] = bench_load_path(ops, dev)
