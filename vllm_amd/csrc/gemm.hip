@@ -9,7 +9,8 @@ namespace w4a16 {
 
 // Planner overrides for tuning runs exist only in builds made with -DW4A16_TUNING: W4A16_SPLITS, W4A16_TN and
 // W4A16_KIND (0 general, 1 decode, 2 prefill, 3 64-row, 5 64-row with in-workgroup K split) force the K split count, the
-// decode tile width and the kernel kind; W4A16_DEBUG=1 prints the chosen plan to stderr, =2 every candidate.
+// decode tile width and the kernel kind, W4A16_NW (4 or 8) the wavefronts per workgroup of the 16-row kernels;
+// W4A16_DEBUG=1 prints the chosen plan to stderr, =2 every candidate.
 // The shipped library reads no environment variable and prints nothing.
 #ifdef W4A16_TUNING
 static int env_int(const char* name, int dflt) {
