@@ -234,6 +234,32 @@ def test_moe_gemm_tail_tiles_split_on_the_device(dev, m, foreign):
     assert int(ws.abs().sum()) == 0
 
 
+def test_moe_gemm_more_than_65535_tiles(dev):
+    """5000 blocks of 8 slots x 16 column tiles: the 16-row kernel's tile index spills into the grid's third dimension
+    (workgroups past the last tile leave at once, after their share of the zero-fill side job)."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    m, topk, e, bs, k, n = 40000, 1, 2, 8, 128, 2048
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, 128, torch.float16, False, False, seed=90)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).half()
+    ids = rand_topk(m, topk, e, seed=6)
+    tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7))
+    s, x, t = moe_align_block_size(ids.to(dev), bs, e)
+    ws = marlin_make_workspace_new(dev, 4)
+    out = ops.moe_wna16_marlin_gemm(
+        a.to(dev), None, mq.to(dev), None, ms.to(dev), None, mz.to(dev), gi.to(dev), perm.to(dev), ws, s, x, t,
+        tw.to(dev), moe_block_size=bs, top_k=topk, mul_topk_weights=True, is_ep=False, b_q_type=scalar_types.uint4b8,
+        size_m=m, size_n=n, size_k=k, is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False).cpu()
+    flat = ids.flatten().long()
+    for ex in range(e):
+        rows = torch.nonzero(flat == ex).flatten()
+        ref = (a[rows].float() @ layers[ex].w_ref.float()) * tw.flatten()[rows].unsqueeze(1)
+        mtr = gr.error_metrics(out[rows], ref)
+        assert mtr["max_rel"] <= 2e-2 and mtr["mean_rel"] < 0.04, (ex, mtr)
+
+
 def test_moe_gemm_skips_foreign_experts_and_bias(dev):
     """expert_ids = -1 blocks are left untouched (expert parallelism); per-expert bias is added."""
     import vllm_amd.ops as ops

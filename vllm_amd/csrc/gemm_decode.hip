@@ -56,6 +56,9 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   //   plain:   x = split, y + 65535 z = tile                       (the splits of a tile are neighbours)
   //   xcd_map: x = tile % 8, y = split, z = tile / 8               (consecutive workgroups go round the eight XCDs, so
   //            all splits of a tile share one XCD's L2)
+  // (every workgroup of the grid takes its share of the side job, also one that has no tile)
+  if constexpr (MOE)
+    zero_fill_side_job(p, (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x, gridDim.x * gridDim.y * gridDim.z);
   int tile, split;
   if (p.xcd_map) {
     tile = blockIdx.z * 8 + blockIdx.x;
@@ -70,8 +73,6 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     ct = tile % p.ncp;
     mt = tile / p.ncp;
   }
-  if constexpr (MOE)
-    zero_fill_side_job(p, (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x, gridDim.x * gridDim.y * gridDim.z);
 
   const uint32_t* Bq = p.B;
   const uint16_t* Sc = (const uint16_t*)p.S;
