@@ -258,6 +258,13 @@ def test_moe_gemm_more_than_65535_tiles(dev):
         ref = (a[rows].float() @ layers[ex].w_ref.float()) * tw.flatten()[rows].unsqueeze(1)
         mtr = gr.error_metrics(out[rows], ref)
         assert mtr["max_rel"] <= 2e-2 and mtr["mean_rel"] < 0.04, (ex, mtr)
+    # the same launch through the fused operator with a buffer to clear on the side: every 16-byte piece is cleared
+    fill = torch.full((3 * 1024 * 1024 + 40,), 1.0, dtype=torch.float16, device=dev)
+    c = torch.empty(m * topk, n, dtype=torch.float16, device=dev)
+    ops.moe_marlin_gemm_fused(a.to(dev), c, mq.to(dev), None, ms.to(dev), None, mz.to(dev), gi.to(dev), perm.to(dev), ws, s,
+                              x, t, tw.to(dev), bs, topk, True, scalar_types.uint4b8, m, n, k, True, False, 0, fill)
+    assert int(torch.count_nonzero(fill)) == 0
+    assert torch.equal(c.cpu(), out)
 
 
 def test_moe_gemm_skips_foreign_experts_and_bias(dev):
