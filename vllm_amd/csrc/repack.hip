@@ -119,6 +119,53 @@ __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restr
   }
 }
 
+// The same for layers of at least 512 columns: a workgroup walks 16 k-tiles of a 512-column span, reads every source
+// row's 256 contiguous bytes with 16-byte loads (the next k-tile's are in flight while this one is assembled) and
+// stores 16 bytes per thread; thread t makes the four words (w = 0..3) of Marlin thread t % 32 in n-tile t / 32.
+__global__ __launch_bounds__(256) void awq_repack_wide_kernel(const uint32_t* __restrict__ in,
+                                                              uint32_t* __restrict__ out, int size_k,
+                                                              int size_n, int kt_per_wg) {
+  using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) uint32_t tile[16][64];  // 16 rows x 64 words (512 columns)
+  const int t = threadIdx.x;
+  const int ncol0 = blockIdx.x * 512;
+  const int ncols = min(512, size_n - ncol0);  // a multiple of 64
+  const int kt_begin = blockIdx.y * kt_per_wg, kt_end = min(kt_begin + kt_per_wg, size_k / 16);
+  const int row = t >> 4, cw4 = (t & 15) * 4;
+  const bool ld_on = cw4 * 8 < ncols;
+  const uint32_t* src = in + (size_t)row * (size_n >> 3) + (ncol0 >> 3) + cw4;
+  const size_t kt_stride = (size_t)16 * (size_n >> 3);
+  const int nt = t >> 5, th = t & 31;
+  const bool st_on = nt * 64 < ncols;
+  const int r = 2 * (th & 3), c = th >> 2;
+  const int nib = ((c & 1) << 2) | (c >> 1);  // {0,4,1,5,2,6,3,7}[c]
+  u32x4 cur = {0, 0, 0, 0};
+  if (ld_on && kt_begin < kt_end) cur = *(const u32x4*)(src + kt_begin * kt_stride);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    u32x4 nxt = {0, 0, 0, 0};
+    if (ld_on && kt + 1 < kt_end) nxt = *(const u32x4*)(src + (kt + 1) * kt_stride);
+    __syncthreads();  // the previous k-tile's LDS reads are done
+    if (ld_on) *(u32x4*)&tile[row][cw4] = cur;
+    __syncthreads();
+    if (st_on) {
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int kk = r + kDK[j];
+          const uint32_t sw = tile[kk][nt * 8 + 2 * w + ((j >> 1) & 1)];
+          word |= ((sw >> (4 * nib)) & 0xFu) << (4 * j);
+        }
+        o[w] = word;
+      }
+      *(u32x4*)(out + (size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 8 + nt) * 128 + th * 4) = o;
+    }
+    cur = nxt;
+  }
+}
+
 // 8-bit variant (uint8b128): output int32 [K/16, 4N]; per k-tile and n-tile 256 words; word
 // nt*256 + th*8 + 2w + half holds the bytes q[k0 + {0, 8, 1, 9}[j], 64nt + 16w + c + 8 half], j = 0..3
 // (gptq_marlin_repack.cu:119-203 with num_bits = 8).  One thread per output word; load-time only, so the
@@ -306,6 +353,16 @@ extern "C" int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out
   if (num_bits == 8) {
     const unsigned blocks = (unsigned)ceil_div(size_k / 16 * 4 * size_n, 256);
     repack8_kernel<true, false><<<blocks, 256, 0, (hipStream_t)stream>>>(b_q_weight, nullptr, out, (int)size_k, (int)size_n);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
+  if (size_n >= 512 && ((uintptr_t)b_q_weight & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    // k-tiles per workgroup: as many as leave about 2048 workgroups (between 2 and 16)
+    const int64_t units = (size_k / 16) * ceil_div(size_n, 512);
+    int kt_per_wg = (int)(units / 2048);
+    kt_per_wg = kt_per_wg < 2 ? 2 : kt_per_wg > KT_PER_WG ? KT_PER_WG : kt_per_wg;
+    dim3 grid((unsigned)ceil_div(size_n, 512), (unsigned)ceil_div(size_k / 16, kt_per_wg));
+    awq_repack_wide_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k, (int)size_n, kt_per_wg);
     W4A16_HIP(hipGetLastError());
     return 0;
   }
