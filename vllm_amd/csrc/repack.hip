@@ -21,6 +21,11 @@ namespace w4a16 {
 __device__ __constant__ const int kDK[8] = {0, 8, 0, 8, 1, 9, 1, 9};
 // k-tiles one workgroup of the 4-bit repack kernels walks through (16 KB of output per workgroup)
 constexpr int KT_PER_WG = 16;
+// ... of the 512-column kernels: as many as leave about 2048 workgroups (between 2 and 16)
+static int wide_kt_per_wg(int64_t size_k, int64_t size_n) {
+  const int64_t kt = (size_k / 16) * ((size_n + 511) / 512) / 2048;
+  return kt < 2 ? 2 : kt > KT_PER_WG ? KT_PER_WG : (int)kt;
+}
 
 // GPTQ source: word (r, n), nibble i = q[8r + i, n].  Without perm a k-tile is two source rows.
 template <bool HAS_PERM>
@@ -78,6 +83,53 @@ __global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __rest
   }
   out[(size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 2 + nt) * 128 + th * 4 + w] = word;
   }
+  }
+}
+
+// GPTQ source without a row permutation, layers of at least 512 columns: a workgroup walks kt_per_wg k-tiles of a
+// 512-column span, reads the two source rows of a k-tile (2 KB contiguous each) with 16-byte loads, the next k-tile's in
+// flight while this one is assembled, and stores 16 bytes per thread: thread t makes the four words (w = 0..3) of Marlin
+// thread t % 32 in n-tile t / 32.
+__global__ __launch_bounds__(256) void gptq_repack_wide_kernel(const uint32_t* __restrict__ in,
+                                                               uint32_t* __restrict__ out, int size_k,
+                                                               int size_n, int kt_per_wg) {
+  using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) uint32_t tile[2][512];
+  const int t = threadIdx.x;
+  const int ncol0 = blockIdx.x * 512;
+  const int ncols = min(512, size_n - ncol0);  // a multiple of 64
+  const int kt_begin = blockIdx.y * kt_per_wg, kt_end = min(kt_begin + kt_per_wg, size_k / 16);
+  const int row = t >> 7, c4 = (t & 127) * 4;
+  const bool ld_on = c4 < ncols;
+  const uint32_t* src = in + (size_t)row * size_n + ncol0 + c4;
+  const size_t kt_stride = (size_t)2 * size_n;
+  const int nt = t >> 5, th = t & 31;
+  const bool st_on = nt * 64 < ncols;
+  const int r = 2 * (th & 3), c = th >> 2;
+  u32x4 cur = {0, 0, 0, 0};
+  if (ld_on && kt_begin < kt_end) cur = *(const u32x4*)(src + kt_begin * kt_stride);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    u32x4 nxt = {0, 0, 0, 0};
+    if (ld_on && kt + 1 < kt_end) nxt = *(const u32x4*)(src + (kt + 1) * kt_stride);
+    __syncthreads();  // the previous k-tile's LDS reads are done
+    if (ld_on) *(u32x4*)&tile[row][c4] = cur;
+    __syncthreads();
+    if (st_on) {
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int kk = r + kDK[j];
+          const uint32_t sw = tile[kk >> 3][nt * 64 + 16 * w + c + ((j >> 1) & 1) * 8];
+          word |= ((sw >> (4 * (kk & 7))) & 0xFu) << (4 * j);
+        }
+        o[w] = word;
+      }
+      *(u32x4*)(out + (size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 8 + nt) * 128 + th * 4) = o;
+    }
+    cur = nxt;
   }
 }
 
@@ -336,6 +388,13 @@ extern "C" int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
     W4A16_HIP(hipGetLastError());
     return 0;
   }
+  if (!perm && size_n >= 512 && size_n % 4 == 0 && ((uintptr_t)b_q_weight & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    const int kt_per_wg = wide_kt_per_wg(size_k, size_n);
+    dim3 wgrid((unsigned)ceil_div(size_n, 512), (unsigned)ceil_div(size_k / 16, kt_per_wg));
+    gptq_repack_wide_kernel<<<wgrid, 256, 0, s>>>(b_q_weight, out, (int)size_k, (int)size_n, kt_per_wg);
+    W4A16_HIP(hipGetLastError());
+    return 0;
+  }
   dim3 grid((unsigned)ceil_div(size_n, 128), (unsigned)ceil_div(size_k / 16, KT_PER_WG));
   if (perm)
     gptq_repack_kernel<true><<<grid, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n);
@@ -357,10 +416,7 @@ extern "C" int w4a16_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out
     return 0;
   }
   if (size_n >= 512 && ((uintptr_t)b_q_weight & 15) == 0 && ((uintptr_t)out & 15) == 0) {
-    // k-tiles per workgroup: as many as leave about 2048 workgroups (between 2 and 16)
-    const int64_t units = (size_k / 16) * ceil_div(size_n, 512);
-    int kt_per_wg = (int)(units / 2048);
-    kt_per_wg = kt_per_wg < 2 ? 2 : kt_per_wg > KT_PER_WG ? KT_PER_WG : kt_per_wg;
+    const int kt_per_wg = wide_kt_per_wg(size_k, size_n);
     dim3 grid((unsigned)ceil_div(size_n, 512), (unsigned)ceil_div(size_k / 16, kt_per_wg));
     awq_repack_wide_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k, (int)size_n, kt_per_wg);
     W4A16_HIP(hipGetLastError());
