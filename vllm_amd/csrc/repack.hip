@@ -133,6 +133,67 @@ __global__ __launch_bounds__(256) void gptq_repack_wide_kernel(const uint32_t* _
   }
 }
 
+// GPTQ source with a row permutation (act-order), layers of at least 512 columns: as above, but a k-tile gathers its 16
+// rows through perm (row perm[k] lives in source word row perm[k] / 8, nibble perm[k] % 8).  The workgroup's slice of
+// perm is read into LDS once; the 16 source rows' 2 KB pieces of the next k-tile are in flight (eight 16-byte loads
+// per thread) while this one is assembled.
+__global__ __launch_bounds__(256) void gptq_repack_perm_wide_kernel(const uint32_t* __restrict__ in,
+                                                                    const int32_t* __restrict__ perm,
+                                                                    uint32_t* __restrict__ out, int size_k,
+                                                                    int size_n, int kt_per_wg) {
+  using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) uint32_t tile[16][512];
+  __shared__ int src_rows[KT_PER_WG * 16];
+  const int t = threadIdx.x;
+  const int ncol0 = blockIdx.x * 512;
+  const int ncols = min(512, size_n - ncol0);  // a multiple of 64
+  const int kt_begin = blockIdx.y * kt_per_wg, kt_end = min(kt_begin + kt_per_wg, size_k / 16);
+  if (t < (kt_end - kt_begin) * 16) src_rows[t] = perm[kt_begin * 16 + t];
+  __syncthreads();
+  const int rh = t >> 7, c4 = (t & 127) * 4;
+  const bool ld_on = c4 < ncols;
+  const uint32_t* src = in + ncol0 + c4;
+  const int nt = t >> 5, th = t & 31;
+  const bool st_on = nt * 64 < ncols;
+  const int r = 2 * (th & 3), c = th >> 2;
+  u32x4 cur[8], nxt[8];
+  auto load = [&](u32x4* dst, int kt) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      dst[i] = u32x4{0, 0, 0, 0};
+      if (ld_on && kt < kt_end) dst[i] = *(const u32x4*)(src + (size_t)(src_rows[(kt - kt_begin) * 16 + 2 * i + rh] >> 3) * size_n);
+    }
+  };
+  load(cur, kt_begin);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    load(nxt, kt + 1);
+    __syncthreads();  // the previous k-tile's LDS reads are done
+    if (ld_on) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *(u32x4*)&tile[2 * i + rh][c4] = cur[i];
+    }
+    __syncthreads();
+    if (st_on) {
+      const int* rows = src_rows + (kt - kt_begin) * 16;
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int kk = r + kDK[j];
+          const uint32_t sw = tile[kk][nt * 64 + 16 * w + c + ((j >> 1) & 1) * 8];
+          word |= ((sw >> (4 * (rows[kk] & 7))) & 0xFu) << (4 * j);
+        }
+        o[w] = word;
+      }
+      *(u32x4*)(out + (size_t)kt * (2 * size_n) + (size_t)(blockIdx.x * 8 + nt) * 128 + th * 4) = o;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cur[i] = nxt[i];
+  }
+}
+
 // AWQ source: word (k, cw), nibble t = q[k, 8*cw + {0,2,4,6,1,3,5,7}[t]]  =>  column 8*cw + j sits
 // in nibble {0,4,1,5,2,6,3,7}[j].
 __global__ __launch_bounds__(256) void awq_repack_kernel(const uint32_t* __restrict__ in,
@@ -388,10 +449,13 @@ extern "C" int w4a16_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
     W4A16_HIP(hipGetLastError());
     return 0;
   }
-  if (!perm && size_n >= 512 && size_n % 4 == 0 && ((uintptr_t)b_q_weight & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+  if (size_n >= 512 && size_n % 4 == 0 && ((uintptr_t)b_q_weight & 15) == 0 && ((uintptr_t)out & 15) == 0) {
     const int kt_per_wg = wide_kt_per_wg(size_k, size_n);
     dim3 wgrid((unsigned)ceil_div(size_n, 512), (unsigned)ceil_div(size_k / 16, kt_per_wg));
-    gptq_repack_wide_kernel<<<wgrid, 256, 0, s>>>(b_q_weight, out, (int)size_k, (int)size_n, kt_per_wg);
+    if (perm)
+      gptq_repack_perm_wide_kernel<<<wgrid, 256, 0, s>>>(b_q_weight, perm, out, (int)size_k, (int)size_n, kt_per_wg);
+    else
+      gptq_repack_wide_kernel<<<wgrid, 256, 0, s>>>(b_q_weight, out, (int)size_k, (int)size_n, kt_per_wg);
     W4A16_HIP(hipGetLastError());
     return 0;
   }
