@@ -166,3 +166,24 @@ def test_support_queries_and_layer_checks():
     import torch
     assert mu.marlin_moe_intermediate_size(torch.empty(8, 256, 57344), torch.empty(8, 896, 8192)) == 14336
     assert mu.marlin_make_workspace(4096, torch.device("cpu")).shape == (1024,)
+
+
+def test_moe_block_size_rule():
+    """Blocks of 16 slots while an expert's share of the slots stays below ~1.25 blocks (sooner for experts of a few MB),
+    blocks of 64 from there on; never 8, 32 or 48.  The quantity is the reference's (tokens * topk / experts,
+    fused_marlin_moe.py:279-282); the thresholds are this library's."""
+    from vllm_amd.fused_marlin_moe import pick_block_size
+    big, small = 88 << 20, 5 << 20
+    assert pick_block_size(1, 2, 8, big) == 16
+    assert pick_block_size(16, 2, 8, big) == 16           # 4 slots per expert
+    assert pick_block_size(64, 2, 8, big) == 16           # 16
+    assert pick_block_size(79, 2, 8, big) == 16           # 19.75
+    assert pick_block_size(80, 2, 8, big) == 64           # 20
+    assert pick_block_size(4096, 2, 8, big) == 64
+    assert pick_block_size(128, 8, 128, small) == 16      # 8 slots per expert
+    assert pick_block_size(223, 8, 128, small) == 16      # 13.9
+    assert pick_block_size(224, 8, 128, small) == 64      # 14
+    assert pick_block_size(224, 8, 128, big) == 16        # the same share with large experts
+    assert pick_block_size(100, 2, 8) == 64               # default: large experts
+    assert all(pick_block_size(t, k, e, b) in (16, 64) for t in (1, 7, 300, 5000) for k in (1, 2, 8) for e in (4, 64, 256)
+               for b in (small, big))
