@@ -90,14 +90,15 @@ def gemm(ops, wtype, a, layer, workspace):
                                 a.shape[0], layer["n"], layer["k"], True, False, True, False)
 
 
-def time_graph(fn_list, reps, warmup, stats=False):
+def time_graph(fn_list, reps, warmup, stats=False, eager_all=True):
     """Capture `fn_list` (a list of zero-arg launch closures) into one HIP graph, replay it `warmup`
     times untimed and `reps` times, every replay between its own pair of events on the launch stream;
-    returns the median seconds/replay (with stats=True: (median, min))."""
+    returns the median seconds/replay (with stats=True: (median, min)).  Before the capture every closure
+    (eager_all=False: only the first) runs once eagerly."""
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
-        for f in fn_list:  # eager warm-up (module load, allocator)
+        for f in (fn_list if eager_all else fn_list[:1]):  # eager warm-up (module load, allocator)
             f()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -122,8 +123,9 @@ def copies_needed(weight_bytes):
     return max(2, -(-512 * 2**20 // weight_bytes) + 1)
 
 
-def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=40, zp=False):
-    """Cold (rotating weight copies) time of one shape; returns dict."""
+def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=40, zp=False, probe=False):
+    """Cold (rotating weight copies) time of one shape; returns dict.  probe=True is the same launch sequence for a
+    profiler run (`--probe-shape`): one eager launch, then the same graph replays, no warm-weights leg."""
     base = layer_fn(k, n, dtype, dev, 1)
     wbytes = base["q"].numel() * 4
     ncopy = min(copies_needed(wbytes), 64)
@@ -135,7 +137,10 @@ def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=4
     err = float((out.float() - ref).abs().max() / ref.abs().max())
     mean_rel = float((out.float() - ref).abs().mean() / ref.abs().mean())
     fns = [(lambda c=copies[i % ncopy]: gemm(ops, wtype, a, c, workspace)) for i in range(max(launches, ncopy))]
-    sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=5, warmup=1, stats=True))
+    sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=5, warmup=1, stats=True, eager_all=not probe))
+    if probe:
+        return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_min": sec_min * 1e6, "launches_timed": 5 * len(fns),
+                "launches_total": 2 + 6 * len(fns), "max_rel_err": err}
     warm = time_graph([lambda: gemm(ops, wtype, a, base, workspace)] * 20, reps=5, warmup=1) / 20
     by, fl = algorithmic_bytes(m, k, n, zp=zp), 2.0 * m * n * k
     del copies
@@ -355,6 +360,38 @@ def bench_other_types(ops, dev, workspace):
     return out
 
 
+def bench_practical_peak(dev):
+    """What a dense 16-bit GEMM reaches on this GPU through the vendor library (torch.matmul -> hipBLASLt), same harness
+    (graph replays on rotating weight copies), on the four M = 4096 shapes: activations [4096, K] times a dense weight
+    stored [K, N] ("nn") or [N, K] ("nt", multiplied as its transpose).  No dequantisation: the practical ceiling that the
+    2.5 PFLOP/s peak translates to for a GEMM of these shapes."""
+    out = {}
+    m = 4096
+    for dt_name, dt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        for name, (k, n) in LAYERS.items():
+            gen = torch.Generator(device=dev).manual_seed(17)
+            a = torch.randn(m, k, device=dev, generator=gen).to(dt)
+            ncopy = min(copies_needed(k * n * 2), 3)
+            row = {}
+            for layout in ("nn", "nt"):
+                shape = (k, n) if layout == "nn" else (n, k)
+                ws = [(torch.randn(shape, device=dev, generator=gen) * 0.02).to(dt) for _ in range(ncopy)]
+                c = torch.empty(m, n, dtype=dt, device=dev)
+                fns = [(lambda w=ws[i % ncopy]: torch.matmul(a, w if layout == "nn" else w.t(), out=c)) for i in range(8)]
+                sec = time_graph(fns, reps=5, warmup=1) / len(fns)
+                row[layout] = {"us": sec * 1e6, "TFLOPs": 2.0 * m * n * k / sec / 1e12}
+                del ws, c
+                torch.cuda.empty_cache()
+            best = max(row.values(), key=lambda r: r["TFLOPs"])
+            out[f"{name}_M4096_{dt_name}"] = {"m": m, "k": k, "n": n, "nn_us": row["nn"]["us"], "nn_TFLOPs": row["nn"]["TFLOPs"],
+                                              "nt_us": row["nt"]["us"], "nt_TFLOPs": row["nt"]["TFLOPs"],
+                                              "best_TFLOPs": best["TFLOPs"], "best_frac_of_peak": best["TFLOPs"] / MFMA_PEAK_TFLOPS}
+            print(f"[detail] dense torch.matmul {name} M=4096 {dt_name}: nn {row['nn']['us']:.1f} us "
+                  f"({row['nn']['TFLOPs']:.0f} TFLOP/s), nt {row['nt']['us']:.1f} us ({row['nt']['TFLOPs']:.0f} TFLOP/s)",
+                  file=sys.stderr, flush=True)
+    return out
+
+
 def _cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -431,12 +468,6 @@ def main():
     ap.add_argument("--probe-moe", type=int, default=0, metavar="T",
                     help="kernel-trace workload: ten calls of the Mixtral-8x7B-shaped fused MoE (8 experts, top-2, uint4b8 "
                          "g128 fp16, random codes) on T tokens; prints no JSON line")
-    ap.add_argument("--issue-probe", action="store_true",
-                    help="MFMA / VALU issue micro-benchmark (independent MFMAs interleaved with 0..6 VALU instructions, "
-                         "one and two wavefronts per SIMD); prints a table, no JSON line")
-    ap.add_argument("--stream-probe", action="store_true",
-                    help="streaming floor of the 16-row kernels on the four layers (a kernel with their loads and no "
-                         "arithmetic); prints a table, no JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1", file=sys.stderr)
@@ -453,14 +484,6 @@ def main():
     workspace = marlin_make_workspace_new(dev)
     m = args.m
 
-    if args.issue_probe:
-        from vllm_amd import issue_probe
-        issue_probe.run(dev)
-        return
-    if args.stream_probe:
-        from vllm_amd import issue_probe
-        issue_probe.stream_floor(dev, LAYERS, time_graph, copies_needed)
-        return
     if args.probe_moe:
         from vllm_amd.fused_marlin_moe import fused_marlin_moe
         e, hid, inter, topk, t = 8, 4096, 14336, 2, args.probe_moe
@@ -473,26 +496,26 @@ def main():
         logits = torch.randn(t, e, device=dev, generator=gen)
         tw, ti = torch.topk(torch.softmax(logits, dim=-1), topk)
         tw, ti = (tw / tw.sum(dim=-1, keepdim=True)).contiguous(), ti.to(torch.int32).contiguous()
-        for _ in range(10):
-            fused_marlin_moe(x, q1, q2, None, None, s1, s2, logits, tw, ti, quant_type_id=scalar_types.uint4b8.id,
-                             global_num_experts=e)
-        torch.cuda.synchronize()
-        print(f"probe-moe done: 10 calls at T={t}, {int(ti.unique().numel())} experts hit", file=sys.stderr)
+        call = lambda: fused_marlin_moe(x, q1, q2, None, None, s1, s2, logits, tw, ti, quant_type_id=scalar_types.uint4b8.id,
+                                        global_num_experts=e)
+        sec = time_graph([call] * 4, reps=5, warmup=1, eager_all=False) / 4
+        print(f"probe-moe done: 1 eager call + 6 replays of 4 calls at T={t}, {int(ti.unique().numel())} experts hit, "
+              f"{sec * 1e6:.1f} us per call (median replay)", file=sys.stderr)
         return
     if args.probe_shape:
+        # the launch sequence of the `detail` row of the same shape (graph replays on rotating weight copies), so that a
+        # kernel trace of this run averages over the launches that row times
         name, pm, kind = args.probe_shape.split(":")
         k, n = LAYERS[name]
+        pm = int(pm)
         if kind == "awq_bf16":
-            base, wt, dt = make_awq_layer(ops, k, n, torch.bfloat16, dev, 1), scalar_types.uint4, torch.bfloat16
+            r = bench_shape(ops, scalar_types.uint4, lambda *a: make_awq_layer(ops, *a), pm, k, n, torch.bfloat16, dev,
+                            workspace, launches=8 if pm >= 2048 else 40, zp=True, probe=True)
         else:
-            base, wt, dt = make_gptq_layer(ops, k, n, torch.float16, dev, 1), scalar_types.uint4b8, torch.float16
-        ncopy = min(copies_needed(base["q"].numel() * 4), 16)
-        copies = [base] + [clone_weights(base, 100 + i) for i in range(ncopy - 1)]
-        a = torch.randn(int(pm), k, generator=torch.Generator().manual_seed(2)).to(dt).to(dev)
-        for i in range(2 * ncopy):
-            gemm(ops, wt, a, copies[i % ncopy], workspace)
-        torch.cuda.synchronize()
-        print(f"probe-shape done: {2 * ncopy} launches of {name} M={pm} {kind}", file=sys.stderr)
+            r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_layer(ops, *a), pm, k, n, torch.float16, dev,
+                            workspace, launches=8 if pm >= 2048 else 40, probe=True)
+        print(f"probe-shape done: {name} M={pm} {kind}: {r['launches_total']} launches, the last {r['launches_timed']} "
+              f"event-timed at {r['us']:.2f} us per launch (median replay; min {r['us_min']:.2f})", file=sys.stderr)
         return
 
     # ---- headline: one step = the four decode GEMMs, weights rotated over `nsets` full sets
@@ -635,6 +658,15 @@ def main():
             "workload": "llama3-8b linears at M=4096, bf16, AWQ uint4 + uint4 zero points g128 (qkv, o, gate_up, down), "
                         "time-weighted over the four layers",
             "per_layer_frac": {k: round(v["mfma_frac"], 3) for k, v in pf.items()}}
+        pk = bench_practical_peak(dev)
+        result["practical_peak"] = {
+            "what": "dense 16-bit GEMM through torch.matmul (hipBLASLt), no dequantisation, same shapes and harness; "
+                    "nn = weight stored [K, N], nt = stored [N, K]",
+            "unit": "TFLOP/s", "per_shape": pk,
+            "bf16_time_weighted_TFLOPs": sum(2.0 * v["m"] * v["n"] * v["k"] for kk, v in pk.items() if kk.endswith("bf16")) /
+                                         sum(min(v["nn_us"], v["nt_us"]) for kk, v in pk.items() if kk.endswith("bf16")) / 1e6,
+            "w4a16_bf16_awq_vs_dense_bf16": {name: round(pf[f"{name}_M4096"]["TFLOPs"] / pk[f"{name}_M4096_bf16"]["best_TFLOPs"], 3)
+                                             for name in LAYERS}}
         if args.table:
             with open(args.table, "w") as f:
                 json.dump(detail, f, indent=1)

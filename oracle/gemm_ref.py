@@ -15,7 +15,7 @@ are all part of what is checked:
                         unpack nibbles, (q-8)*s or (q-z)*s group-broadcast)
   gemm_ref(a, w)        fp32 matmul (+ bias), result in fp32
 
-Pinned by (tests/test_oracle_gemm.py): dequant_marlin(repack(x)) == w_ref of the
+Pinned by (tests/test_oracle_quant.py, the dequantisation section): dequant_marlin(repack(x)) == w_ref of the
 quantizer bit-for-bit for every (type, group, act-order) combination;
 dequant_checkpoint == w_ref likewise; fp32 matmul is torch's.
 """

@@ -458,3 +458,31 @@ def test_fused_marlin_moe_with_bias(dev):
             act = torch.nn.functional.silu(h[:inter].float()).to(dtype) * h[inter:]
             ref[t] += float(tw[t, j]) * (act.float() @ l2[ex].w_ref.float() + b2[ex].float()).to(dtype).float()
     torch.testing.assert_close(out.cpu().float(), ref, atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("bs", [16, 48])
+def test_moe_gemm_never_uses_memory_past_sorted_ids(dev, bs):
+    """sorted_token_ids of the usual length numel + E * (block - 1), not a multiple of the block size, as an exact-size
+    view in front of slot ids that look valid: the launch's last, never-live block must not pick them up, and the result
+    must equal the one computed from a tensor of its own."""
+    import vllm_amd.ops as ops
+    from vllm_amd.marlin_utils import marlin_make_workspace_new
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    from vllm_amd.scalar_type import scalar_types
+    m, topk, e, k, n = 16, 2, 8, 256, 192
+    layers, mq, ms, mz, gi, perm = make_experts(e, k, n, 128, torch.float16, False, False, seed=10)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).half().to(dev)
+    ids = rand_topk(m, topk, e, seed=6).to(dev)
+    tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7)).to(dev)
+    s, x, t = moe_align_block_size(ids, bs, e)
+    assert s.numel() % bs != 0
+    big = torch.zeros(s.numel() + 4 * bs, dtype=torch.int32, device=dev)   # id 0 behind the end: a valid-looking slot
+    big[:s.numel()] = s
+    ws = marlin_make_workspace_new(dev, 4)
+    call = lambda sorted_ids: ops.moe_wna16_marlin_gemm(
+        a, None, mq.to(dev), None, ms.to(dev), None, None, None, None, ws, sorted_ids, x, t, tw, moe_block_size=bs,
+        top_k=topk, mul_topk_weights=True, is_ep=False, b_q_type=scalar_types.uint4b8, size_m=m, size_n=n, size_k=k,
+        is_k_full=True, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
+    want = call(s)
+    got = call(big[:s.numel()])
+    assert torch.equal(got, want)

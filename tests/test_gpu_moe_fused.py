@@ -147,3 +147,53 @@ def test_fused_marlin_moe_expert_parallel_fused_path(dev):
     mask = torch.isin(ti, torch.tensor(local))
     ref = mr.torch_experts(a, w1, w2, tw * mask, ti)
     torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-2, rtol=0)
+
+
+@pytest.mark.parametrize("scales", [(1e-6, 1e-6), (1.0, 3e-4), (1e-5, 5e-5), (6e-5, -6.1e-5), (300.0, 1e-6)])
+@pytest.mark.parametrize("dtype_variant", ["gptq_f16_g128", "gptq_bf16_chan"])
+def test_top2_sum_epilogue_rounding_on_tiny_and_mixed_rows(dev, scales, dtype_variant):
+    """The fused top-2 sum adds rounded 16-bit rows with packed 16-bit atomic adds; moe_sum adds them in fp32 and rounds.
+    Both are the correctly rounded sum of two 16-bit numbers as long as the atomic unit rounds to nearest even and keeps
+    subnormals: rows scaled into the subnormal range of fp16, rows whose two terms are many binades apart, and terms that
+    nearly cancel, must give the same bits."""
+    import vllm_amd.ops as ops
+    m, topk, e, bs, k, n = 64, 2, 4, 16, 256, 192
+    dtype, _, tw, align, w, ws = _setup(dev, m, topk, e, bs, dtype_variant, k, n, seed=21)
+    tw = torch.empty(m, topk)
+    tw[:, 0], tw[:, 1] = scales
+    tw = (tw * (1 + torch.rand(m, topk, generator=torch.Generator().manual_seed(8)) / 8)).to(dev)
+    a = (torch.randn(m * topk, k, generator=torch.Generator().manual_seed(9)) / 4).to(dtype).to(dev)
+    y = _plain(ops, a, w, ws, align, tw, bs, 1, True, m * topk, n, k)
+    want = torch.empty(m, n, dtype=dtype, device=dev)
+    ops.moe_sum(y.view(m, topk, n), want)
+    got = torch.zeros(m, n, dtype=dtype, device=dev)
+    _fused(ops, a, got, w, ws, align, tw, bs, 1, True, m * topk, n, k, sum_top_k=2)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert float(want.float().abs().max()) > 0
+    if dtype == torch.float16 and max(abs(s) for s in scales) < 1e-4:
+        sub = (want.float().abs() < 6.1e-5) & (want != 0)          # subnormal results are what this case is about
+        assert float(sub.float().mean()) > 0.5
+
+
+@pytest.mark.parametrize("inter,strided", [(96, False), (128, True), (96, True)])
+def test_fused_marlin_moe_falls_back_when_the_fused_epilogues_do_not_apply(dev, inter, strided):
+    """An intermediate size that is not a multiple of 64 (no gate / up n-tile pairing) and a strided `output` must take
+    the separate-launch path instead of failing the operator's argument checks."""
+    from vllm_amd.fused_marlin_moe import fused_marlin_moe
+    from oracle import moe_ref as mr
+    dtype, e, topk, m, k = torch.float16, 4, 2, 50, 256
+    l1, q1, s1, _, _, _ = make_experts(e, k, 2 * inter, 128, dtype, False, False, seed=500)
+    l2, q2, s2, _, _, _ = make_experts(e, inter, k, 32, dtype, False, False, seed=600)
+    g = torch.Generator().manual_seed(13)
+    a = (torch.randn(m, k, generator=g) / 10).to(dtype)
+    tw, ti = torch.topk(torch.softmax(torch.randn(m, e, generator=g), dim=-1), topk)
+    out = torch.zeros(m, 2 * k, dtype=dtype, device=dev)[:, ::2] if strided else None
+    res = fused_marlin_moe(a.to(dev), q1.to(dev), q2.to(dev), None, None, s1.to(dev), s2.to(dev), None, tw.to(dev),
+                           ti.to(torch.int32).to(dev), quant_type_id=l1[0].type_id, global_num_experts=e, output=out)
+    if strided:
+        assert res is out
+    w1 = torch.stack([l.w_ref.t() for l in l1])
+    w2 = torch.stack([l.w_ref.t() for l in l2])
+    ref = mr.torch_experts(a, w1, w2, tw, ti)
+    torch.testing.assert_close(res.cpu().float(), ref.float(), atol=5e-2, rtol=0)

@@ -87,12 +87,13 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   // five in a row, before it can address its weights and activations (short-K expert GEMMs live only a few of them)
   int id_0 = 0, id_a0 = 0, id_a1 = 0, id_t = 0, moe_e = 0, moe_ntp = 0;
   if constexpr (MOE) {
-    const int* ids = p.sorted_ids + mt * p.moe_bs;
-    const int last = p.moe_bs - 1;
-    id_0 = ids[0];
-    id_a0 = ids[min(ar, last)];
-    id_a1 = ids[min(ar + 8, last)];
-    id_t = ids[min(tr, last)];
+    // (the last block of the grid may reach past the end of sorted_ids, whose length need not be a multiple of the block
+    //  size; such a block is never live, and its loads are clamped onto the array's last element)
+    const int first = mt * p.moe_bs, last = p.moe_bs - 1, end = p.n_sorted - 1;
+    id_0 = p.sorted_ids[min(first, end)];
+    id_a0 = p.sorted_ids[min(first + min(ar, last), end)];
+    id_a1 = p.sorted_ids[min(first + min(ar + 8, last), end)];
+    id_t = p.sorted_ids[min(first + min(tr, last), end)];
     moe_ntp = *p.ntpp;
     moe_e = p.expert_ids[mt];
   }

@@ -105,12 +105,13 @@ __global__ __launch_bounds__(NW * 64, 2) void skinny_kernel(const KParams p) {
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) id_a[mb] = 0;
   if (p.moe) {
-    const int* ids = p.sorted_ids + mt * p.moe_bs;
-    const int last = p.moe_bs - 1;
-    id_0 = ids[0];
+    // (the last block of the grid may reach past the end of sorted_ids, whose length need not be a multiple of the block
+    //  size; such a block is never live, and its loads are clamped onto the array's last element)
+    const int first = mt * p.moe_bs, last = p.moe_bs - 1, end = p.n_sorted - 1;
+    id_0 = p.sorted_ids[min(first, end)];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) id_a[mb] = ids[min(mb * 16 + am, last)];
-    id_t = ids[min(tr, last)];
+    for (int mb = 0; mb < MB; ++mb) id_a[mb] = p.sorted_ids[min(first + min(mb * 16 + am, last), end)];
+    id_t = p.sorted_ids[min(first + min(tr, last), end)];
     moe_ntp = *p.ntpp;
     moe_e = p.expert_ids[mt];
   }

@@ -101,9 +101,12 @@ def _run_experts(x: torch.Tensor, ex: _Experts, rt: _Routing, weight_on_input: b
     act = inter_buf.view(-1)[:slots * n].view(slots, n) if inter_buf is not None else torch.empty((slots, n), device=dev, dtype=dt)
     # what the GEMM launches can take over: SiLU-and-mul in GEMM1's epilogue whenever the default activation is asked
     # for; the top-k sum in GEMM2's epilogue for two terms (a sum of two does not depend on their order)
-    act_fused = activation == "silu" and activation_func is default_activation_func
-    sum_fused = reduce_topk and moe_sum is None and rt.topk == 2
-    direct = not reduce_topk or (moe_sum is None and rt.topk == 1)   # GEMM2 writes the result rows themselves
+    # (the fused activation pairs gate and up n-tiles of 64 columns: the intermediate size must be a multiple of 64; the
+    #  GEMM writes rows of a contiguous output: a strided `out` takes the separate-launch path and a final copy)
+    act_fused = activation == "silu" and activation_func is default_activation_func and n % 64 == 0
+    out_ok = out is None or out.is_contiguous()
+    sum_fused = reduce_topk and moe_sum is None and rt.topk == 2 and out_ok
+    direct = (not reduce_topk or (moe_sum is None and rt.topk == 1)) and out_ok   # GEMM2 writes the result rows themselves
     if (sum_fused or direct) and out is None:
         out = torch.empty((m if reduce_topk else slots, k), device=dev, dtype=dt)
     needs_zero = sum_fused or (direct and rt.expert_parallel)    # rows of experts on other ranks are never written
@@ -134,9 +137,17 @@ def _run_experts(x: torch.Tensor, ex: _Experts, rt: _Routing, weight_on_input: b
     y = _gemm(ex, 1, rt, act, y, slots, k, n, 1, not weight_on_input)
     if out is None:
         out = torch.empty((m, k), device=dev, dtype=dt)
+    if not reduce_topk:          # (a strided `out` for the unreduced rows)
+        out.copy_(y)
+        return out
     y3 = y.view(m, rt.topk, k)
     if moe_sum is None:
-        ops.moe_sum(y3, out)
+        if out.is_contiguous():
+            ops.moe_sum(y3, out)
+        else:
+            dense = torch.empty((m, k), device=dev, dtype=dt)
+            ops.moe_sum(y3, dense)
+            out.copy_(dense)
         return out
     return moe_sum(y3, out)
 
