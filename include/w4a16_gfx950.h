@@ -165,11 +165,15 @@ int w4a16_marlin_gemm(const w4a16_gemm_args* args, void* stream);
  * harnesses that forbid hipMalloc).  No counterpart in the reference, whose op allocates c_tmp and a_tmp itself
  * (gptq_marlin.cu:751-763).  args->c_tmp, args->workspace and args->workspace_len are ignored: split-K partial
  * tiles, the column-gathered copy of A (act-order) and the arrival counters live in a buffer of
- * W4A16_STATIC_SCRATCH_BYTES inside the library's own device memory, one per GPU, held until the process ends.
+ * W4A16_STATIC_SCRATCH_BYTES (+ 16 KiB of counters) inside the library's own device memory: resident on every GPU of
+ * every process that loads the library, whether or not this entry point is ever called, until the process ends.
  * A problem that needs more scratch than that (w4a16_gemm_scratch_bytes says how much) fails with W4A16_EINVAL and a
  * message; nothing is launched then.  The call allocates and frees nothing.  All calls on one GPU share that GPU's
  * buffer: calls that overlap in time on one GPU (two streams, two host threads) race and must be serialised by the
- * caller.  Inputs and the output are the caller's, as in w4a16_marlin_gemm, and results are identical to it. */
+ * caller.  Inputs and the output are the caller's, as in w4a16_marlin_gemm, and results are identical to those of
+ * w4a16_marlin_gemm called with a workspace of 4096 counters (the launch plan looks at the workspace length: a shorter
+ * workspace can rule out a K split).  MoE calls whose 64-row tiles may split K on the device ask for the buffer's
+ * whole size in partial tiles when the tile count is large; add the act-order copy of A and they are refused. */
 #define W4A16_STATIC_SCRATCH_BYTES (64u << 20)
 int w4a16_marlin_gemm_static(const w4a16_gemm_args* args, void* stream);
 
