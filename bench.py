@@ -86,8 +86,9 @@ def clone_weights(layer, seed):
 
 def gemm(ops, wtype, a, layer, workspace):
     e = torch.empty(0, dtype=torch.int32, device=a.device)
-    return ops.gptq_marlin_gemm(a, None, layer["q"], None, layer["s"], None, layer["zp"], e, e, workspace, wtype,
-                                a.shape[0], layer["n"], layer["k"], True, False, True, False)
+    return ops.gptq_marlin_gemm(a, None, layer["q"], None, layer["s"], None, layer["zp"], layer.get("g_idx", e),
+                                layer.get("perm", e), workspace, wtype, a.shape[0], layer["n"], layer["k"], True, False,
+                                True, False)
 
 
 def time_graph(fn_list, reps, warmup, stats=False, eager_all=True):
@@ -137,10 +138,11 @@ def bench_shape(ops, wtype, layer_fn, m, k, n, dtype, dev, workspace, launches=4
     err = float((out.float() - ref).abs().max() / ref.abs().max())
     mean_rel = float((out.float() - ref).abs().mean() / ref.abs().mean())
     fns = [(lambda c=copies[i % ncopy]: gemm(ops, wtype, a, c, workspace)) for i in range(max(launches, ncopy))]
-    sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=5, warmup=1, stats=True, eager_all=not probe))
-    if probe:
-        return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_min": sec_min * 1e6, "launches_timed": 5 * len(fns),
-                "launches_total": 2 + 6 * len(fns), "max_rel_err": err}
+    if probe:  # more replays, so that the two eager launches in front weigh nothing in a trace's average
+        sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=11, warmup=1, stats=True, eager_all=False))
+        return {"m": m, "k": k, "n": n, "us": sec * 1e6, "us_min": sec_min * 1e6, "launches_timed": 11 * len(fns),
+                "launches_total": 2 + 12 * len(fns), "max_rel_err": err}
+    sec, sec_min = (t / len(fns) for t in time_graph(fns, reps=5, warmup=1, stats=True))
     warm = time_graph([lambda: gemm(ops, wtype, a, base, workspace)] * 20, reps=5, warmup=1) / 20
     by, fl = algorithmic_bytes(m, k, n, zp=zp), 2.0 * m * n * k
     del copies
@@ -463,7 +465,7 @@ def main():
                     help="counter-collection workload: plain device copies of known size (calibration) followed by "
                          "eager launches of the headline GEMMs on cold weights; prints no JSON line")
     ap.add_argument("--probe-shape", type=str, default="",
-                    help="counter-collection workload for one shape, LAYER:M:KIND with KIND gptq_f16 or awq_bf16 "
+                    help="counter-collection workload for one shape, LAYER:M:KIND with KIND gptq_f16, gptq_act_f16 or awq_bf16 "
                          "(e.g. gate_up:4096:awq_bf16): a few eager launches on rotating weight copies; prints no JSON line")
     ap.add_argument("--probe-moe", type=int, default=0, metavar="T",
                     help="kernel-trace workload: ten calls of the Mixtral-8x7B-shaped fused MoE (8 experts, top-2, uint4b8 "
@@ -511,6 +513,9 @@ def main():
         if kind == "awq_bf16":
             r = bench_shape(ops, scalar_types.uint4, lambda *a: make_awq_layer(ops, *a), pm, k, n, torch.bfloat16, dev,
                             workspace, launches=8 if pm >= 2048 else 40, zp=True, probe=True)
+        elif kind == "gptq_act_f16":
+            r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_actorder_layer(ops, *a), pm, k, n, torch.float16,
+                            dev, workspace, launches=16, probe=True)
         else:
             r = bench_shape(ops, scalar_types.uint4b8, lambda *a: make_gptq_layer(ops, *a), pm, k, n, torch.float16, dev,
                             workspace, launches=8 if pm >= 2048 else 40, probe=True)

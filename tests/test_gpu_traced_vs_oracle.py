@@ -37,6 +37,7 @@ def test_compiled_gemm_matches_oracle(dev, mode, group, m):
     dtype = torch.float16 if (m + group) % 2 else torch.bfloat16
     layer, wtype, dev_ops = _operands(dev, mode, group, dtype, seed=m + (group & 255))
     ws = marlin_make_workspace_new(dev)
+    torch._dynamo.reset()   # every case compiles the same code object anew: start from an empty cache
     fn = torch.compile(lambda x: _gemm(x, None, dev_ops, ws, wtype.id), fullgraph=True, backend="aot_eager", dynamic=False)
     a = torch.randn(m, K, generator=torch.Generator().manual_seed(m)).to(dtype)
     out = fn(a.to(dev))
@@ -54,7 +55,8 @@ def test_compiled_gemm_dynamic_m_matches_oracle(dev, mode, group):
     layer, wtype, dev_ops = _operands(dev, mode, group, dtype, seed=77)
     ws = marlin_make_workspace_new(dev)
     torch._dynamo.reset()
-    fn = torch.compile(lambda x: _gemm(x, None, dev_ops, ws, wtype.id), fullgraph=True, backend="aot_eager", dynamic=True)
+    type_id = int(wtype.id)   # (computed outside the traced function: only M is meant to be symbolic)
+    fn = torch.compile(lambda x: _gemm(x, None, dev_ops, ws, type_id), fullgraph=True, backend="aot_eager", dynamic=True)
     for m in (5, 48, 19, 130, 2):
         a = torch.randn(m, K, generator=torch.Generator().manual_seed(m)).to(dtype)
         out = fn(a.to(dev))
@@ -113,6 +115,7 @@ def test_compiled_apply_weights_matches_oracle(dev, mode):
     kern = MarlinLinearKernel(cfg, "qweight", "scales", "qzeros" if mode == "awq" else None,
                               "g_idx" if mode == "gptq_act_order" else None)
     kern.process_weights_after_loading(layer)
+    torch._dynamo.reset()
     compiled = torch.compile(lambda x, b: kern.apply_weights(layer, x, b), fullgraph=True, backend="aot_eager", dynamic=False)
     for m in (3, 40, 200):
         g = torch.Generator().manual_seed(m)

@@ -88,3 +88,71 @@ def test_static_scratch_gemm_rejects_oversized(dev):
     assert b"static buffer" in lib.w4a16_last_error()
     torch.cuda.synchronize()
     assert float(c.min()) == 7.0 and float(c.max()) == 7.0
+
+
+def _moe_args(lib_mod, a, c, q, s, g_idx, perm, ws, align, tw, bs, topk, m, n, k, e):
+    sorted_ids, expert_ids, post = align
+    args = _args(lib_mod, a, c, {"q": q, "s": s}, m, n, k, s.shape[1], ws, None, None, g_idx, perm, torch.float16)
+    args.flags |= lib_mod.F_MOE | lib_mod.F_MUL_TOPK_WEIGHTS
+    args.sorted_token_ids, args.expert_ids = sorted_ids.data_ptr(), expert_ids.data_ptr()
+    args.num_tokens_past_padded, args.topk_weights = post.data_ptr(), tw.data_ptr()
+    args.n_sorted = min(sorted_ids.numel(), expert_ids.numel() * bs)
+    args.moe_block_size, args.top_k, args.num_experts = bs, topk, e
+    return args
+
+
+@pytest.mark.parametrize("bs,ms", [(16, (24, 5)), (64, (600, 200))])
+def test_static_scratch_moe_gemm_matches(dev, bs, ms):
+    """The MoE mode through the entry point that allocates nothing: blocks of 16 (16-row kernel) and blocks of 64 (64-row
+    kernel, whose K split of the tail tiles is decided on the device and keeps its partial tiles in the scratch)."""
+    from test_gpu_moe import make_experts, rand_topk
+    from vllm_amd import _lib
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    lib = _lib.load()
+    e, topk, k, n = 4, 2, 4096, 512
+    layers, mq, ms_, _, _, _ = make_experts(e, k, n, 128, torch.float16, False, False, seed=70)
+    q, s = mq.to(dev), ms_.to(dev)
+    ws = torch.zeros(4096, dtype=torch.int32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    for m in ms:
+        print(f"static scratch MoE case bs={bs} m={m}", flush=True)
+        a = (torch.randn(m, k, generator=torch.Generator().manual_seed(m)) / 4).half().to(dev)
+        ids = rand_topk(m, topk, e, seed=m).to(dev)
+        tw = torch.rand(m, topk, generator=torch.Generator().manual_seed(7)).to(dev)
+        align = moe_align_block_size(ids, bs, e)
+        want = torch.zeros(m * topk, n, dtype=torch.float16, device=dev)
+        got = torch.zeros(m * topk, n, dtype=torch.float16, device=dev)
+        args = _moe_args(_lib, a, want, q, s, None, None, ws, align, tw, bs, topk, m, n, k, e)
+        need = lib.w4a16_gemm_scratch_bytes(ctypes.byref(args))
+        assert 0 <= need <= _lib.STATIC_SCRATCH_BYTES
+        c_tmp = torch.empty(max(need // 4, 1), dtype=torch.float32, device=dev)
+        args.c_tmp = c_tmp.data_ptr()
+        _lib.check(lib.w4a16_marlin_gemm(ctypes.byref(args), stream))
+        sargs = _moe_args(_lib, a, got, q, s, None, None, None, align, tw, bs, topk, m, n, k, e)
+        _lib.check(lib.w4a16_marlin_gemm_static(ctypes.byref(sargs), stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        assert float(want.float().abs().max()) > 0 and int(ws.abs().sum()) == 0
+
+
+def test_static_scratch_moe_act_order_is_refused_when_it_does_not_fit(dev):
+    """MoE with act-order needs one gathered row of A per sorted slot on top of the partial tiles: a call whose total
+    exceeds the static buffer is refused with the message, and nothing is launched."""
+    from vllm_amd import _lib
+    from vllm_amd.moe_align_block_size import moe_align_block_size
+    lib = _lib.load()
+    e, topk, k, n, m, bs = 8, 2, 14336, 4096, 2048, 64
+    q = torch.zeros(e, k // 16, 2 * n, dtype=torch.int32, device=dev)
+    s = torch.ones(e, k // 128, n, dtype=torch.float16, device=dev)
+    idx = torch.arange(k, dtype=torch.int32, device=dev).repeat(e, 1).contiguous()
+    g_idx = (idx // 128).contiguous()
+    a = torch.zeros(m, k, dtype=torch.float16, device=dev)
+    ids = (torch.arange(m * topk, device=dev, dtype=torch.int32) % e).view(m, topk).contiguous()
+    tw = torch.ones(m, topk, device=dev)
+    align = moe_align_block_size(ids, bs, e)
+    c = torch.full((m * topk, n), 7.0, dtype=torch.float16, device=dev)
+    args = _moe_args(_lib, a, c, q, s, g_idx, idx, None, align, tw, bs, topk, m, n, k, e)
+    rc = lib.w4a16_marlin_gemm_static(ctypes.byref(args), ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == -1 and b"static buffer" in lib.w4a16_last_error()
+    torch.cuda.synchronize()
+    assert float(c.min()) == 7.0 and float(c.max()) == 7.0

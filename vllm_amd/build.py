@@ -13,6 +13,11 @@ LIB_PATH = os.path.join(HERE, LIB_NAME)
 
 SOURCES = ["c_api.hip", "repack.hip", "gemm.hip", "gemm_skinny.hip", "gemm_decode.hip", "gemm_fat.hip", "gemm_mid.hip", "gemm_kq.hip", "moe_glue.hip"]
 
+# The 16-row kernel takes the values in front of its first loads as leading scalar arguments; with this option the first
+# 14 dwords of a kernel's argument block arrive in SGPRs when a wavefront starts (gfx950 firmware loads them while it
+# dispatches; the compiler keeps a fallback prologue that loads them itself).
+FILE_FLAGS = {"gemm_decode.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
+
 # packed-fp32 VALU forms are switched off for every device compile of this library
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -43,7 +48,7 @@ def build(verbose: bool = False, extra_flags: tuple = (), check_hazards: bool = 
         for s in srcs:
             o = s[:-4] + ".o"
             objs.append(o)
-            cmd = [hipcc_path()] + [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags)
+            cmd = [hipcc_path()] + [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags) + FILE_FLAGS.get(os.path.basename(s), [])
             if os.path.basename(s) in ASM_MFMA_SOURCES:
                 # intermediate files land beside the object: build it in the scratch folder and move it afterwards
                 o_build = os.path.join(tmpdir, os.path.basename(o))

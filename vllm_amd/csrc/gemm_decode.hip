@@ -35,8 +35,19 @@ struct DecodeCfg {
 
 // MOE: the launch walks MoE blocks (slot ids, expert ids, fused epilogues); the dense instantiations carry none of that
 // code, which shortens the chain of argument loads in front of a small layer's first weight load
+// The leading scalar arguments repeat fields of `p`: the file is compiled with kernel-argument preloading, which hands
+// the first 14 dwords of the argument block to a wavefront in SGPRs when it starts.  Everything in front of the first
+// weight and activation loads (tile and K range of the workgroup, the operands' addresses) is computed from those
+// registers alone, so a small layer's first loads do not wait for a fetch of the argument block from memory (a round
+// trip as long as the weight load itself when the launch comes from a graph and the block is cold).
+//   eNcpX: column tiles, bit 30 set for the XCD-aware grid; eKpsG: k-steps per split, (group_shift + 1) << 24
 template <int DT, bool ZP, bool CHANNEL, int TN, int DNW, bool MOE>
-__global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
+__global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const uint32_t* eB, const void* eA, const void* eS,
+                                                             int64_t eLda, int eN, int eKpsG, int eTotal, int eTiles,
+                                                             int eNcpX, int eM, const KParams p) {
+  const int eNcp = eNcpX & 0x3fffffff;
+  const bool eXcd = (eNcpX >> 30) & 1;
+  const int eKps = eKpsG & 0xffffff, eGroupShift = (eKpsG >> 24) - 1;
   constexpr int W = TN / 32;  // Marlin words per lane and k-tile: 4 (128-bit load) or 2 (64-bit load)
   constexpr bool HI_TRICK = (DT == DT_F16) && !ZP;
   constexpr int RS = DecodeCfg<TN>::RS;
@@ -60,22 +71,22 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   if constexpr (MOE)
     zero_fill_side_job(p, (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x, gridDim.x * gridDim.y * gridDim.z);
   int tile, split;
-  if (p.xcd_map) {
+  if (eXcd) {
     tile = blockIdx.z * 8 + blockIdx.x;
     split = blockIdx.y;
   } else {
     tile = blockIdx.z * 65535 + blockIdx.y;
     split = blockIdx.x;
-    if (tile >= p.tiles) return;
+    if (tile >= eTiles) return;
   }
   int ct = tile, mt = 0;  // column tile, m-tile
-  if (p.ncp != p.tiles) {
-    ct = tile % p.ncp;
-    mt = tile / p.ncp;
+  if (eNcp != eTiles) {
+    ct = tile % eNcp;
+    mt = tile / eNcp;
   }
 
-  const uint32_t* Bq = p.B;
-  const uint16_t* Sc = (const uint16_t*)p.S;
+  const uint32_t* Bq = eB;
+  const uint16_t* Sc = (const uint16_t*)eS;
   const uint32_t* Zp = p.Z;
   const uint16_t* bias = (const uint16_t*)p.bias;
   // activation loads: lane -> row (lane >> 3) [+ 8 for the second load], 16-byte piece (lane & 7) of the
@@ -108,7 +119,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
       }
     } else {
       const int gr = mt * 16 + r;
-      if (gr < p.M) src = dst = gr;
+      if (gr < eM) src = dst = gr;
     }
   };
   const uint16_t* arow[2];
@@ -120,7 +131,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     for (int i = 0; i < 2; ++i) {
       int src, dst;
       tile_row_ids(ar + 8 * i, i ? id_a1 : id_a0, src, dst);
-      arow[i] = (const uint16_t*)p.A + (int64_t)(src >= 0 ? src : src0) * p.lda + ap * 8;
+      arow[i] = (const uint16_t*)eA + (int64_t)(src >= 0 ? src : src0) * eLda + ap * 8;
     }
   }
   if (threadIdx.x < 16) {
@@ -138,8 +149,8 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   }
 
   // ---- this wavefront's stages (pairs of k-steps)
-  const int st_b = split * p.ksteps_per_split / 2;
-  const int st_e = min(st_b + p.ksteps_per_split / 2, p.total_ksteps / 2);
+  const int st_b = split * eKps / 2;
+  const int st_e = min(st_b + eKps / 2, eTotal / 2);
   const int per = (st_e - st_b + DNW - 1) / DNW;
   const int w_b = min(st_b + wv * per, st_e), w_e = min(w_b + per, st_e);
   const int nst = w_e - w_b;
@@ -147,10 +158,10 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   // n-tile this lane reads (TN=128: 2ct+h, TN=64: ct); a missing second n-tile (N/64 odd) aliases n-tile 0
   int nt;
   if (TN == 128)  // (fused SiLU-and-mul: gate n-tile ct paired with the up n-tile of the same output columns)
-    nt = (MOE && p.act) ? (h ? (p.N >> 7) + ct : ct) : ((2 * ct + h) * 64 < p.N ? 2 * ct + h : 0);
+    nt = (MOE && p.act) ? (h ? (eN >> 7) + ct : ct) : ((2 * ct + h) * 64 < eN ? 2 * ct + h : 0);
   else
     nt = ct;
-  const int64_t b_row = (int64_t)p.N * 2;  // words per k-tile row
+  const int64_t b_row = (int64_t)eN * 2;  // words per k-tile row
   // TN=128: words th*4 .. +4 of the n-tile, th = 4c+g.  TN=64: words th*4 + 2h .. +2.
   const uint32_t* bp = Bq + (int64_t)nt * 128 + (4 * c + g) * 4 + (TN == 64 ? 2 * h : 0) + (int64_t)(4 * w_b) * b_row;
   // scales of the lane's columns: permuted position 8c + j, j = 2w + half; TN=64 covers w = 2h, 2h+1 only
@@ -165,11 +176,11 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   const uint32_t* slab_rd = slab + (lane & 15) * A_ROW + g;
 
   // rows 8..15 of the tile exist?  (otherwise their activation loads are skipped)
-  const bool rows_hi = MOE ? (p.moe_bs > 8) : (mt * 16 + 8 < p.M);
+  const bool rows_hi = MOE ? (p.moe_bs > 8) : (mt * 16 + 8 < eM);
   // scale group of an absolute stage index (channel-wise scales: pseudo-groups of 128 K rows, so that the raw partial
   // sums, biased by E * sum(a), stay small next to fp32's 24 bits whatever the activations' mean)
   auto group_of = [&](int sidx) {
-    return CHANNEL ? (sidx >> 1) : (p.group_shift >= 0 ? (2 * sidx) >> p.group_shift : (2 * sidx) / p.group_ksteps);
+    return CHANNEL ? (sidx >> 1) : (eGroupShift >= 0 ? (2 * sidx) >> eGroupShift : (2 * sidx) / p.group_ksteps);
   };
   struct Stage {
     bvec b[4];   // k-tiles 4s .. 4s+3
@@ -192,8 +203,8 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     const int gi = group_of(sidx);
     s.gi = gi;
     if (sidx == w_b || gi != group_of(sidx - 1)) {  // uniform: only the first stage of a group carries its scales
-      if (!CHANNEL) s.sc = *(const bvec*)(sp + (int64_t)gi * p.N);
-      if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (p.N >> 3)];
+      if (!CHANNEL) s.sc = *(const bvec*)(sp + (int64_t)gi * eN);
+      if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (eN >> 3)];
     }
     const uint32_t* q = bp + (int64_t)(4 * (sidx - w_b)) * b_row;
 #pragma unroll
@@ -337,7 +348,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   const int fc = (t & 31) * CPT;        // first column inside the tile
   const int fpos = (TN == 128) ? fc + (fc >= 64 ? 8 : 0) : fc + (fc >= 32 ? 8 : 0);
   const int ncol = ct * TN + fc;
-  const bool fcol_ok = ncol < p.N;
+  const bool fcol_ok = ncol < eN;
   const bool single = p.splits == 1;
   float* my_part = p.ctmp + ((int64_t)tile * p.splits + split) * (16 * TN);
 
@@ -383,7 +394,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
   if (MOE && TN == 128 && p.act) {
     if (act_lane) {
       col_consts(ct * 64 + fc, cs, bs);
-      col_consts((p.N >> 1) + ct * 64 + fc, cu, bu);
+      col_consts((eN >> 1) + ct * 64 + fc, cu, bu);
     }
   } else if (fcol_ok) {
     col_consts(ncol, cs, bs);
@@ -408,7 +419,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
     } else {
       const uint32_t o = pack2<DT>(v[0], v[1]);
       if (MOE && p.sum_div > 0) {
-        uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * p.N + ncol;
+        uint16_t* dst = (uint16_t*)p.C + (int64_t)(crow / p.sum_div) * eN + ncol;
         if constexpr (DT == DT_F16) {
           typedef _Float16 h2 __attribute__((ext_vector_type(2)));
           __builtin_amdgcn_global_atomic_fadd_v2f16((h2*)dst, __builtin_bit_cast(h2, o));
@@ -417,7 +428,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
           __builtin_amdgcn_global_atomic_fadd_v2bf16((s2*)dst, __builtin_bit_cast(s2, o));
         }
       } else {
-        *(uint32_t*)((uint16_t*)p.C + (int64_t)crow * p.N + ncol) = o;
+        *(uint32_t*)((uint16_t*)p.C + (int64_t)crow * eN + ncol) = o;
       }
     }
   };
@@ -509,7 +520,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const KParams p) {
 }
 
 // ------------------------------------------------------------------------------------ host side
-typedef void (*decode_fn)(const KParams);
+typedef void (*decode_fn)(const uint32_t*, const void*, const void*, int64_t, int, int, int, int, int, int, const KParams);
 
 template <int DT, int TN, int NW, bool MOE>
 static decode_fn pick5(bool zp, bool channel) {
@@ -552,7 +563,8 @@ int launch_decode(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) 
     const unsigned gy = pl.tiles < 65535 ? (unsigned)pl.tiles : 65535u;
     grid = dim3((unsigned)pl.splits, gy, (unsigned)((pl.tiles + 65534) / 65535));
   }
-  hipLaunchKernelGGL(fn, grid, dim3(nw * 64), smem, stream, p);
+  hipLaunchKernelGGL(fn, grid, dim3(nw * 64), smem, stream, p.B, p.A, p.S, p.lda, p.N, p.ksteps_per_split | ((p.group_shift + 1) << 24), p.total_ksteps,
+                     p.tiles, p.ncp | (p.xcd_map ? (1 << 30) : 0), p.M, p);
   W4A16_HIP(hipGetLastError());
   return 0;
 }
