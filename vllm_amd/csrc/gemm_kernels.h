@@ -138,6 +138,27 @@ __device__ __forceinline__ void store_row4_silu_mul(const KParams& p, int crow, 
 // through to the device-coherent level) and read back with agent-scope loads (sc1: never served from a
 // non-coherent line), 8 bytes at a time.  The writer waits for its stores (s_waitcnt) before it counts
 // itself as arrived; the reader is whoever sees the last arrival.
+//
+// Why the last arriver reads complete partial tiles, instruction by instruction (16-row kernels, gemm_decode.hip /
+// gemm_skinny.hip epilogue):
+//   1. every thread of a writing workgroup issues its partial sums as `global_store_dwordx2 ... sc1`: the store is
+//      performed at the device-coherent level, not left dirty in the XCD's L2;
+//   2. `s_waitcnt vmcnt(0)` (__builtin_amdgcn_s_waitcnt(0)) in every thread: vmcnt only drops when the memory system has
+//      acknowledged the store, i.e. when it is performed at that level, so after the wait the thread's words are visible
+//      to any later sc1 load of any compute unit;
+//   3. `s_barrier`: all threads of the workgroup have passed step 2 before thread 0 goes on;
+//   4. thread 0 executes `global_atomic_inc ... sc0` at agent scope on the tile's counter: a read-modify-write performed
+//      at the same coherent level, issued after (program order + the barrier) every store of its workgroup was
+//      acknowledged.  Read-modify-writes on one address are totally ordered, so exactly one workgroup reads the value
+//      splits - 1, and at that point every other workgroup's increment, hence (steps 2-3) every other workgroup's stores,
+//      have been performed;
+//   5. the returned value reaches the other threads through LDS and a second `s_barrier`; their `global_load_dwordx2
+//      ... sc1` are issued after that barrier, cannot be served from a stale line of the compute unit's or the XCD's
+//      cache, and therefore return the performed stores.
+// What this does not use: a release/acquire fence pair (buffer_wbl2 / buffer_inv).  The argument rests on sc1 accesses
+// being performed at one common level in issue order per thread after an acknowledged wait, which is how the ISA defines
+// them, not on the HIP memory model's fences; tests/test_gpu_splitk_stress.py runs thousands of back-to-back launches of
+// these paths and compares every result bit for bit.
 __device__ __forceinline__ void store_coherent2(float* ptr, float f0, float f1) {
   using u64 = unsigned long long;
   const u64 a = (u64)__builtin_bit_cast(uint32_t, f0) | ((u64)__builtin_bit_cast(uint32_t, f1) << 32);
