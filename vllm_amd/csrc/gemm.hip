@@ -315,7 +315,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
 
   // The decode kernel handles 16-row tiles whose scale groups span whole stages of 64 K rows.
   const bool decode_shape = !general_only && pl.gm != GM_GIDX && pl.total_ksteps % 2 == 0 &&
-                            (pl.gm == GM_CHANNEL || pl.group_ksteps % 2 == 0) && forced_kind != 0;
+                            (pl.gm == GM_CHANNEL || (pl.group_ksteps % 2 == 0 && pow2_group)) && forced_kind != 0;
 
   // Launch-shape choice by a small cost model (microseconds) fitted to MI355X measurements of these
   // kernels.  One 8-wavefront workgroup sustains ~33 GB/s on a 128-column strip and ~20 GB/s on a 64-column

@@ -25,7 +25,11 @@ namespace w4a16 {
 // Wavefronts per workgroup: 8, or 4 when a launch has several workgroups per compute unit in turn: two 4-wavefront
 // workgroups share a compute unit (same registers and loads in flight as one of 8), so one's prologue and
 // epilogue latencies run under the other's weight stream.
-constexpr int DD = 3;   // stages (of two k-steps) in flight per wavefront
+// Stages (of two k-steps) in flight per wavefront.  Two: with three to five the kernel is slower on every layer of the
+// decode step (a wavefront's loads are consumed in order, the eight wavefronts of a workgroup already keep ~64 KB per
+// compute unit in flight, and every further stage costs 20-29 registers and lengthens the prologue); with one, 64-column
+// tiles lose a few per cent.
+constexpr int DD = 2;
 
 template <int TN>
 struct DecodeCfg {
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const uint32_t* eB,
     nt = ct;
   const int64_t b_row = (int64_t)eN * 2;  // words per k-tile row
   // TN=128: words th*4 .. +4 of the n-tile, th = 4c+g.  TN=64: words th*4 + 2h .. +2.
-  const uint32_t* bp = Bq + (int64_t)nt * 128 + (4 * c + g) * 4 + (TN == 64 ? 2 * h : 0) + (int64_t)(4 * w_b) * b_row;
+  const uint32_t* bnext = Bq + (int64_t)nt * 128 + (4 * c + g) * 4 + (TN == 64 ? 2 * h : 0) + (int64_t)(4 * w_b) * b_row;
   // scales of the lane's columns: permuted position 8c + j, j = 2w + half; TN=64 covers w = 2h, 2h+1 only
   const uint16_t* sp = Sc + (int64_t)nt * 64 + 8 * c + (TN == 64 ? 4 * h : 0);
   const uint32_t* zp = ZP ? Zp + nt * 8 + c : nullptr;
@@ -179,9 +183,9 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const uint32_t* eB,
   const bool rows_hi = MOE ? (p.moe_bs > 8) : (mt * 16 + 8 < eM);
   // scale group of an absolute stage index (channel-wise scales: pseudo-groups of 128 K rows, so that the raw partial
   // sums, biased by E * sum(a), stay small next to fp32's 24 bits whatever the activations' mean)
-  auto group_of = [&](int sidx) {
-    return CHANNEL ? (sidx >> 1) : (eGroupShift >= 0 ? (2 * sidx) >> eGroupShift : (2 * sidx) / p.group_ksteps);
-  };
+  // (grouped scales: the host only picks this kernel for power-of-two groups of at least one stage)
+  auto group_of = [&](int sidx) { return CHANNEL ? (sidx >> 1) : ((2 * sidx) >> eGroupShift); };
+  const int gmask = CHANNEL ? 1 : (((1 << eGroupShift) - 1) >> 1);  // stage index bits inside a group
   struct Stage {
     bvec b[4];   // k-tiles 4s .. 4s+3
     u32x4 a[2];  // rows ar, ar+8
@@ -202,11 +206,12 @@ __global__ __launch_bounds__(DNW * 64, 2) void decode_kernel(const uint32_t* eB,
     }
     const int gi = group_of(sidx);
     s.gi = gi;
-    if (sidx == w_b || gi != group_of(sidx - 1)) {  // uniform: only the first stage of a group carries its scales
+    if (sidx == w_b || (sidx & gmask) == 0) {  // uniform: only the first stage of a group carries its scales
       if (!CHANNEL) s.sc = *(const bvec*)(sp + (int64_t)gi * eN);
       if (ZP) s.zq = zp[(int64_t)(CHANNEL ? 0 : gi) * (eN >> 3)];
     }
-    const uint32_t* q = bp + (int64_t)(4 * (sidx - w_b)) * b_row;
+    const uint32_t* q = bnext;  // (stages are issued in order: a running pointer instead of a 64-bit product per stage)
+    bnext += 4 * b_row;
 #pragma unroll
     for (int t = 0; t < 4; ++t) s.b[t] = __builtin_nontemporal_load((const bvec*)(q + t * b_row));
   };
