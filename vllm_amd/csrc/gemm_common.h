@@ -72,7 +72,11 @@ __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
 //  fp16:  value = (1024+q) - zl  |  (1024+16q)/16 - zh , then * s         (all packed-half ops;
 //         every step is exact except the final multiply, so the operand equals
 //         half(q - z) * half(s) rounded once — the reference's w_ref)
-//  bf16:  value = bf16_rne( fma(float(q), s, c) ),  c = -z*s exact in fp32  (single rounding)
+//  bf16:  the nibbles are turned into the same exact fp16 pairs, (1024+q) and (1024+16q), and one mixed-precision
+//         FMA per value (v_fma_mix_f32: fp16 x fp32 + fp32 -> fp32) gives (q - z) * s in fp32:
+//         fma(1024+q, s, -(1024+z) s)  |  fma(1024+16q, s/16, -(64+z) s).  The constants are exact in fp32 (at most
+//         11 + 8 bits) and so is the result (at most 5 + 8 bits), which v_cvt_pk_bf16_f32 then rounds once:
+//         bf16_rne((q - z) * s), the reference's w_ref.
 template <int DT>
 struct ColConst;
 
@@ -85,7 +89,9 @@ struct ColConst<DT_F16> {
 template <>
 struct ColConst<DT_BF16> {
   float s0, s1;  // scale of half 0 / half 1
-  float c0, c1;  // -z*s
+  float c0, c1;  // -(1024+z)*s
+  float h0, h1;  // s/16
+  float d0, d1;  // -(64+z)*s
 };
 
 // raw: (s_half0, s_half1) packed 16-bit pair as loaded; z0/z1: integer zero points (8 for uint4b8)
@@ -100,8 +106,15 @@ __device__ __forceinline__ ColConst<DT> make_col_const(uint32_t s_pair, uint32_t
   } else {
     cc.s0 = UNIT_SCALE ? 1.0f : bf16_lo_f32(s_pair);
     cc.s1 = UNIT_SCALE ? 1.0f : bf16_hi_f32(s_pair);
-    cc.c0 = -(float)z0 * cc.s0;
-    cc.c1 = -(float)z1 * cc.s1;
+    // 1024+z as fp32 bits: 2^10 has its ulp at 2^-13, so z sits at bit 13 of the mantissa
+    const float t0 = __builtin_bit_cast(float, 0x44800000u | (z0 << 13));
+    const float t1 = __builtin_bit_cast(float, 0x44800000u | (z1 << 13));
+    cc.c0 = -t0 * cc.s0;
+    cc.c1 = -t1 * cc.s1;
+    cc.h0 = cc.s0 * 0.0625f;
+    cc.h1 = cc.s1 * 0.0625f;
+    cc.d0 = __builtin_fmaf(960.0f, cc.s0, cc.c0);
+    cc.d1 = __builtin_fmaf(960.0f, cc.s1, cc.c1);
   }
   return cc;
 }
@@ -134,23 +147,19 @@ __device__ __forceinline__ void dequant_pair(uint32_t xa, uint32_t xb, const Col
     o1 = u32x4{lo(ya, zl1, s1), hi(ya, zh1, s1), lo(yb, zl1, s1), hi(yb, zh1, s1)};
   } else {
     // nibble j of a word: j=0 (k0,n0) 1 (k0+8,n0) 2 (k0,n0+8) 3 (k0+8,n0+8) 4..7 same with k0+1
-    auto cvt = [&](uint32_t x, uint32_t& a0, uint32_t& a1, uint32_t& b0, uint32_t& b1) {
-      const uint32_t e = x & 0x0f0f0f0fu;         // bytes: nibbles 0,2,4,6
-      const uint32_t o = (x >> 4) & 0x0f0f0f0fu;  // bytes: nibbles 1,3,5,7
-      const float n0 = (float)(e & 0xff), n2 = (float)((e >> 8) & 0xff), n4 = (float)((e >> 16) & 0xff),
-                  n6 = (float)(e >> 24);
-      const float n1 = (float)(o & 0xff), n3 = (float)((o >> 8) & 0xff), n5 = (float)((o >> 16) & 0xff),
-                  n7 = (float)(o >> 24);
-      a0 = pack_bf16(__builtin_fmaf(n0, cc.s0, cc.c0), __builtin_fmaf(n4, cc.s0, cc.c0));  // (k0,k0+1) half0
-      a1 = pack_bf16(__builtin_fmaf(n1, cc.s0, cc.c0), __builtin_fmaf(n5, cc.s0, cc.c0));  // (k0+8,k0+9) half0
-      b0 = pack_bf16(__builtin_fmaf(n2, cc.s1, cc.c1), __builtin_fmaf(n6, cc.s1, cc.c1));
-      b1 = pack_bf16(__builtin_fmaf(n3, cc.s1, cc.c1), __builtin_fmaf(n7, cc.s1, cc.c1));
+    uint32_t EX = 0x64006400u;
+    asm("" : "+v"(EX));
+    auto lo = [&](uint32_t x, float sf, float cf) {   // nibbles 0 and 4 of x: 1024+q
+      const f16x2 v = as_h2((x & 0x000f000fu) | EX);
+      return pack_bf16(__builtin_fmaf((float)v.x, sf, cf), __builtin_fmaf((float)v.y, sf, cf));
     };
-    uint32_t p0, p1, p2, p3, q0, q1, q2, q3;
-    cvt(xa, p0, p1, q0, q1);
-    cvt(xb, p2, p3, q2, q3);
-    o0 = u32x4{p0, p1, p2, p3};
-    o1 = u32x4{q0, q1, q2, q3};
+    auto hi = [&](uint32_t x, float hf, float df) {   // nibbles 1 and 5 of x: 1024+16q
+      const f16x2 v = as_h2((x & 0x00f000f0u) | EX);
+      return pack_bf16(__builtin_fmaf((float)v.x, hf, df), __builtin_fmaf((float)v.y, hf, df));
+    };
+    const uint32_t ya = xa >> 8, yb = xb >> 8;
+    o0 = u32x4{lo(xa, cc.s0, cc.c0), hi(xa, cc.h0, cc.d0), lo(xb, cc.s0, cc.c0), hi(xb, cc.h0, cc.d0)};
+    o1 = u32x4{lo(ya, cc.s1, cc.c1), hi(ya, cc.h1, cc.d1), lo(yb, cc.s1, cc.c1), hi(yb, cc.h1, cc.d1)};
   }
 }
 
@@ -213,6 +222,30 @@ __device__ __forceinline__ float ubyte_f32(uint32_t x) {
   return f;
 }
 
+// bf16, the two steps of one operand register apart (the prefill kernel issues them between different MFMAs):
+// the exact fp16 pair of nibbles 2*HF + ODD and that + 4 of x, then the two mixed FMAs and the pack.
+template <int HF, int ODD>
+__device__ __forceinline__ uint32_t bf16_piece_halves(uint32_t x) {
+  uint32_t EX = 0x64006400u;
+  asm("" : "+v"(EX));
+  const uint32_t y = HF ? (x >> 8) : x;
+  return (y & (ODD ? 0x00f000f0u : 0x000f000fu)) | EX;
+}
+template <int HF, int ODD>
+__device__ __forceinline__ void bf16_piece_fma(uint32_t halves, const ColConst<DT_BF16>& cc, float& f0, float& f1) {
+  const f16x2 v = as_h2(halves);
+  const float m = ODD ? (HF ? cc.h1 : cc.h0) : (HF ? cc.s1 : cc.s0);
+  const float a = ODD ? (HF ? cc.d1 : cc.d0) : (HF ? cc.c1 : cc.c0);
+  f0 = __builtin_fmaf((float)v.x, m, a);
+  f1 = __builtin_fmaf((float)v.y, m, a);
+}
+template <int HF, int ODD>
+__device__ __forceinline__ uint32_t bf16_piece_pack(uint32_t halves, const ColConst<DT_BF16>& cc) {
+  float f0, f1;
+  bf16_piece_fma<HF, ODD>(halves, cc, f0, f1);
+  return pack_bf16(f0, f1);
+}
+
 // One register (J = 0..7) of what dequant_pair produces: J < 4 -> o0[J], else o1[J - 4].  Lets a caller spread
 // the dequantisation of a Marlin word pair between MFMAs a few instructions at a time.
 template <int DT, bool UNIT_SCALE, int J>
@@ -236,10 +269,7 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t xa, uint32_t xb, cons
     }
     return as_u32(UNIT_SCALE ? v : v * sc);
   } else {
-    // nibbles 2*HF + (Q&1) and that + 4: both sit in byte HF / HF + 2 of the even- or odd-nibble word
-    const uint32_t m = ((Q & 1) ? (x >> 4) : x) & 0x0f0f0f0fu;
-    const float sf = HF ? cc.s1 : cc.s0, cf = HF ? cc.c1 : cc.c0;
-    return pack_bf16(__builtin_fmaf(ubyte_f32<HF>(m), sf, cf), __builtin_fmaf(ubyte_f32<HF + 2>(m), sf, cf));
+    return bf16_piece_pack<HF, Q & 1>(bf16_piece_halves<HF, Q & 1>(x), cc);
   }
 }
 

@@ -166,6 +166,15 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   store_a(0);
   // B operands of the current and of the next k-step (the roles swap every k-step)
   u32x4 ob[2][4][2];
+  // integer 4-bit weights: the dequantisation constants of the four word positions.  A loop iteration covers four
+  // k-steps (128 rows of K), so with groups of 128 rows or more, or one scale per column, they change at most once
+  // per iteration and are kept in registers instead of being rebuilt from the scale and zero-point words every k-step.
+  constexpr bool CONSTS = (BITS == 4 && FP4 == 0 && !ZPF);
+  ColConst<DT> ccs[4];
+  if constexpr (CONSTS) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) ccs[w] = col_const(st[0], w);
+  }
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     if constexpr (ZPF) {
@@ -175,8 +184,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
       const Fp4Scales fs = fp4_scales(st[0], w);
       dequant_pair_fp4<DT>(st[0].b0[w], st[0].b1[w], fs.a0, fs.a1, fs.b0, fs.b1, ob[0][w][0], ob[0][w][1]);
     } else if constexpr (BITS == 4) {
-      const ColConst<DT> cc = col_const(st[0], w);
-      dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], cc, ob[0][w][0], ob[0][w][1]);
+      dequant_pair<DT, UNIT>(st[0].b0[w], st[0].b1[w], ccs[w], ob[0][w][0], ob[0][w][1]);
     } else if constexpr (FP8) {
       dequant_pair8_fp8<DT, UNIT>(word8(st[0], w, 0, 0), word8(st[0], w, 0, 1), word8(st[0], w, 1, 0),
                                   word8(st[0], w, 1, 1), CHANNEL ? 0u : st[0].sc[w], ob[0][w][0], ob[0][w][1]);
@@ -191,32 +199,29 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   // one register of the next k-step's operands (3-5 VALU instructions) is dequantised into ob[CUR ^ 1]; the
   // scheduling barriers keep the compiler from regrouping that into MFMA-only and VALU-only blocks, which would
   // leave the matrix pipe idle during the VALU blocks.
-  auto kstep = [&](auto cur_tag, int buf, int kk, const Stage& nxt) {
+  auto kstep = [&](auto cur_tag, int buf, int kk, const Stage& nxt, auto refresh_tag) {
     constexpr int CUR = decltype(cur_tag)::value;
     const u32x4* abase = (const u32x4*)(lds + buf * (FB_ABUF / 4)) + (kk * FB_MB) * 64 + lane;
     u32x4 af[FB_MB];
 #pragma unroll
     for (int mb = 0; mb < FB_MB; ++mb) af[mb] = abase[mb * 64];
-    // bf16 integer weights: the three dependent stages of one operand register (nibbles -> two floats, two fmas,
-    // one pack) are spread over three consecutive MFMA pairs, so that no VALU instruction reads the result of the
-    // one issued just before it
-    constexpr bool PIPE = (BITS == 4 && FP4 == 0 && !ZPF && DT == DT_BF16);
-    float pc0 = 0.f, pc1 = 0.f, pf0 = 0.f, pf1 = 0.f;
-    auto stage_a = [&](auto p_tag) {  // piece P: nibble bytes -> floats
+    if constexpr (CONSTS && decltype(refresh_tag)::value) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) ccs[w] = col_const(nxt, w);
+    }
+    // bf16 integer weights: the three dependent stages of one operand register (nibbles -> exact fp16 pair, two
+    // mixed FMAs, one pack) are spread over three consecutive MFMA pairs, so that no VALU instruction reads the
+    // result of the one issued just before it
+    constexpr bool PIPE = (CONSTS && DT == DT_BF16);
+    uint32_t ph = 0;
+    float pf0 = 0.f, pf1 = 0.f;
+    auto stage_a = [&](auto p_tag) {  // piece P: nibbles -> (1024+q | 1024+16q) fp16 pair
       constexpr int P = decltype(p_tag)::value, w = P >> 3, J = P & 7, HF = J >> 2, Q = J & 3;
-      const uint32_t x = (Q < 2) ? nxt.b0[w] : nxt.b1[w];
-      const uint32_t m = ((Q & 1) ? (x >> 4) : x) & 0x0f0f0f0fu;
-      pc0 = ubyte_f32<HF>(m);
-      pc1 = ubyte_f32<HF + 2>(m);
+      if constexpr (DT == DT_BF16) ph = bf16_piece_halves<HF, Q & 1>((Q < 2) ? nxt.b0[w] : nxt.b1[w]);
     };
     auto stage_b = [&](auto p_tag) {  // (q - z) * s in fp32, exact
-      constexpr int P = decltype(p_tag)::value, w = P >> 3, HF = (P & 7) >> 2;
-      const ColConst<DT> cc = col_const(nxt, w);
-      if constexpr (DT == DT_BF16) {
-        const float sf = HF ? cc.s1 : cc.s0, cf = HF ? cc.c1 : cc.c0;
-        pf0 = __builtin_fmaf(pc0, sf, cf);
-        pf1 = __builtin_fmaf(pc1, sf, cf);
-      }
+      constexpr int P = decltype(p_tag)::value, w = P >> 3, HF = (P & 7) >> 2, Q = P & 3;
+      if constexpr (DT == DT_BF16) bf16_piece_fma<HF, Q & 1>(ph, ccs[w], pf0, pf1);
     };
     if constexpr (PIPE) {
       stage_a(std::integral_constant<int, 0>{});
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
     }
     auto word = [&](auto w_tag) {
       constexpr int w = decltype(w_tag)::value;
-      const ColConst<DT> cc = col_const(nxt, w);
+      const ColConst<DT>& cc = ccs[w];
       const Fp4Scales fs = fp4_scales(nxt, w);
       uint32_t zs = 0;
       if constexpr (ZPF) zs = as_u32(as_h2(nxt.zf[w]) * as_h2(nxt.sc[w]));
@@ -272,26 +277,41 @@ __global__ __launch_bounds__(256) void fat_kernel(const KParams p) {
   const std::integral_constant<int, 0> even{};
   const std::integral_constant<int, 1> odd{};
 
-  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration
+  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration.  The last k-step of an iteration
+  // dequantises the first k-step of the next 128 rows of K: the constants are rebuilt there, and in the other three
+  // k-steps too when a group is shorter than 128 rows.
+  auto main_loop = [&](auto every_tag) {
+    const std::true_type refresh{};
 #pragma unroll 1
-  for (int c0 = 0; c0 < nchunks; c0 += 2) {
-    const int ks0 = 2 * c0;
-    // chunk c0 in buffer 0
-    load_a(c0 + 1);
-    kstep(even, 0, 0, st[1]);
-    issue(st[0], ks0 + 4);
-    kstep(odd, 0, 1, st[2]);
-    issue(st[1], ks0 + 5);
-    store_a(1);
-    __syncthreads();
-    // chunk c0+1 in buffer 1
-    load_a(c0 + 2);
-    kstep(even, 1, 0, st[3]);
-    issue(st[2], ks0 + 6);
-    kstep(odd, 1, 1, st[0]);
-    issue(st[3], ks0 + 7);
-    store_a(0);
-    __syncthreads();
+    for (int c0 = 0; c0 < nchunks; c0 += 2) {
+      const int ks0 = 2 * c0;
+      // chunk c0 in buffer 0
+      load_a(c0 + 1);
+      kstep(even, 0, 0, st[1], every_tag);
+      issue(st[0], ks0 + 4);
+      kstep(odd, 0, 1, st[2], every_tag);
+      issue(st[1], ks0 + 5);
+      store_a(1);
+      __syncthreads();
+      // chunk c0+1 in buffer 1
+      load_a(c0 + 2);
+      kstep(even, 1, 0, st[3], every_tag);
+      issue(st[2], ks0 + 6);
+      kstep(odd, 1, 1, st[0], refresh);
+      issue(st[3], ks0 + 7);
+      store_a(0);
+      __syncthreads();
+    }
+  };
+  if constexpr (!CONSTS) {
+    main_loop(std::true_type{});
+  } else if constexpr (CHANNEL) {
+    main_loop(std::false_type{});
+  } else {
+    if (p.group_shift < 2)
+      main_loop(std::true_type{});
+    else
+      main_loop(std::false_type{});
   }
 
   // ------------------------------------------------------------------------------ epilogue
