@@ -177,6 +177,7 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
   // a round of 128-row tiles costs 1 (0.6 when its trailing strips are handed to the 64-row kernel); 64-row tiles cost
   // 0.75 with one workgroup per compute unit and 1.15 per pair with two.  (2048 x 4096: 128 tiles of 128 rows leave
   // half the compute units idle, 256 tiles of 64 rows do not: 99 -> 75 us at K = 4096.)
+  const bool kq_types = !general_only && !w8 && a->wtype != W4A16_WTYPE_FE2M1 && !(a->flags & W4A16_F_ZP_FLOAT);
   bool prefer_mid = false;
   if (fat_tiles >= cus / 2 && forced_kind < 0 && mid_ok && !w8) {  // (the unit costs below are the 4-bit kernels')
     const int64_t mt128 = ceil_div(a->size_m, 128), tail = fat_tiles % cus;
@@ -185,6 +186,31 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     const int64_t mid_tiles = ceil_div(a->size_m, 64) * ceil_div(a->size_n, 512), rem = mid_tiles % (2 * cus);
     const double mid_units = 1.15 * (double)(mid_tiles / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.75 : 1.15);
     prefer_mid = mid_units < 0.95 * fat_units;
+  }
+  // 128 x 256 tiles with the K halves inside the workgroup (gemm_kq.hip, MB = 8): the prefill kernel's operand reuse for
+  // problems whose 128 x 512 tiles would leave half the compute units idle.  One round only.
+  {
+    const int64_t tall_tiles = ceil_div(a->size_m, 128) * ceil_div(a->size_n, 256);
+    const bool tall_shape = !moe && kq_types && pow2_group && pl.gm != GM_GIDX && a->size_k % 256 == 0 && a->size_m > 128;
+    const bool tall_pays = tall_tiles <= cus && tall_tiles * 4 >= cus * 3;
+    if (tall_shape && (forced_kind == 6 || (forced_kind < 0 && tall_pays))) {
+      pl.kind = 5;
+      pl.tn = 256;
+      pl.mb = 8;
+      pl.bm = 128;
+      pl.mtiles = (int)ceil_div(a->size_m, 128);
+      pl.ncp = (int)ceil_div(a->size_n, 256);
+      W4A16_CHECK(tall_tiles < (1LL << 31) / 64, "too many tiles");
+      pl.tiles = (int)tall_tiles;
+      pl.splits = 1;
+      pl.kps = pl.total_ksteps;
+      pl.xcd_map = 0;
+      pl.ctmp_bytes = 0;
+      if (debug_plan)
+        fprintf(stderr, "[w4a16] M=%lld N=%lld K=%lld kind=5 (128 x 256) tiles=%d\n", (long long)a->size_m,
+                (long long)a->size_n, (long long)a->size_k, pl.tiles);
+      return 0;
+    }
   }
   if (!moe && fat_ok && pow2_group && a->size_m >= 128 && !prefer_mid && (fat_tiles >= cus / 2 || forced_kind == 2) && a->size_k % 128 == 0 &&
       pl.gm != GM_GIDX && forced_kind != 0 && forced_kind != 1 && forced_kind != 3 && forced_kind != 5) {
@@ -207,9 +233,17 @@ static int make_plan(const w4a16_gemm_args* a, Plan& pl) {
     {
       const int64_t rounds = tiles / cus, tail = tiles - rounds * cus;
       const int64_t strips = ceil_div(tail, (int64_t)pl.mtiles);
-      if (rounds >= 1 && tail > 0 && strips < pl.ncp && strips * ceil_div(a->size_m, 64) <= cus && forced_kind != 2 &&
-          mid_ok)
-        pl.tail_strips = (int)strips;
+      if (rounds >= 1 && tail > 0 && strips < pl.ncp && forced_kind != 2) {
+        // ... or, better, to 128 x 256 tiles whose K halves run on the four wavefronts of one workgroup (the operand reuse
+        // of the prefill kernel, half a round) when those fit one round
+        if (kq_types && a->size_k % 256 == 0 && 2 * strips * pl.mtiles <= cus) {
+          pl.tail_strips = (int)strips;
+          pl.tail_kind = 5;
+        } else if (strips * ceil_div(a->size_m, 64) <= cus && mid_ok) {
+          pl.tail_strips = (int)strips;
+          pl.tail_kind = 3;
+        }
+      }
     }
     return 0;
   }
@@ -434,6 +468,14 @@ static int run_planned(const w4a16_gemm_args* args, Plan& pl, void* stream) {
     head.ncp = pl.ncp - pl.tail_strips;
     head.tiles = head.ncp * pl.mtiles;
     if (int rc = launch_fat(&b, head, (hipStream_t)stream)) return rc;
+    if (pl.tail_kind == 5) {  // 128 x 256 tiles, K halves inside the workgroup
+      tail.kind = 5;
+      tail.tn = 256;
+      tail.ncp = 2 * pl.tail_strips;
+      tail.tiles = tail.mtiles * tail.ncp;
+      tail.strip0 = 2 * head.ncp;
+      return launch_kq(&b, tail, (hipStream_t)stream);
+    }
     tail.kind = 3;
     tail.mb = 4;
     tail.bm = 64;

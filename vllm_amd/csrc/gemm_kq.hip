@@ -17,7 +17,11 @@
 //                kernel's partial bytes for the same number of wavefronts on the problem.
 // Compared with 16-row tiles (which re-read and re-convert the weight strip once per 16 rows) every weight is fetched
 // and dequantised once per 64 rows; compared with the 64 x 512 tile there are 2 x 4 times as many independent streams.
-// Requirements (host-checked): K % 512 == 0 (every quarter runs whole ring periods of 4 k-steps), scales grouped (a
+// A second shape of the same kernel (MB = 8, Q = 2: 4 wavefronts, one per SIMD, 128 rows x 256 columns, K in halves, 256
+// accumulators per lane) serves problems with 128-row tiles that are too few for the prefill kernel's 128 x 512 tiles:
+// every dequantised operand register feeds eight row blocks as in the prefill kernel, and the two K halves are added
+// through LDS instead of through memory.
+// Requirements (host-checked): K % 512 == 0 (Q = 2: K % 256 == 0) (every quarter runs whole ring periods of 4 k-steps), scales grouped (a
 // power-of-two number of k-steps) or channelwise, no per-row g_idx, A's columns already in weight order.
 #include <type_traits>
 
@@ -25,18 +29,19 @@
 
 namespace w4a16 {
 
-constexpr int KQ_MB = 4;     // m-blocks per tile
-constexpr int KQ_BM = 64;    // rows per tile
 constexpr int KQ_TN = 256;   // columns per tile
-constexpr int KQ_Q = 4;      // K-quarters
 constexpr int KQ_D = 4;      // weight k-steps in flight per wavefront
-constexpr int KQ_ABUF = 2 * KQ_MB * 64 * 16;                 // one A buffer of one quarter: 2 k-steps x 4 m-blocks x 64 lanes x 16 B
-constexpr int KQ_SLABS = 8 * 16 * RED_RS * 4;                // eight wavefront slabs of the epilogue
-constexpr int KQ_STAGE = KQ_Q * 2 * KQ_ABUF;
-constexpr int KQ_SMEM = (KQ_STAGE > KQ_SLABS ? KQ_STAGE : KQ_SLABS) + KQ_BM * 4;  // + C row of each tile row
+// MB m-blocks of 16 rows per tile, K cut into Q parts inside the workgroup (2 Q wavefronts)
+constexpr int kq_abuf(int MB) { return 2 * MB * 64 * 16; }  // one A buffer of one K part: 2 k-steps x MB m-blocks x 64 lanes x 16 B
+constexpr int kq_smem(int MB, int Q) {
+  const int stage = Q * 2 * kq_abuf(MB), slabs = 2 * Q * 16 * RED_RS * 4;  // staging rings | the wavefronts' epilogue slabs
+  return (stage > slabs ? stage : slabs) + 16 * MB * 4;                     // + C row of each tile row
+}
 
-template <int DT, bool ZP, bool CHANNEL>
-__global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
+template <int DT, bool ZP, bool CHANNEL, int MB = 4, int Q = 4>
+__global__ __launch_bounds__(128 * Q) void kq_kernel(const KParams p) {
+  static_assert((MB == 4 && Q == 4) || (MB == 8 && Q == 2), "64 x 256 in K quarters or 128 x 256 in K halves");
+  constexpr int KQ_MB = MB, KQ_BM = 16 * MB, KQ_Q = Q, KQ_ABUF = kq_abuf(MB), KQ_SMEM = kq_smem(MB, Q);
   constexpr bool UNIT = CHANNEL;
   extern __shared__ __align__(16) unsigned char smem[];
   int* s_crow = (int*)(smem + KQ_SMEM - KQ_BM * 4);
@@ -50,7 +55,7 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   const int mtiles = (p.M + KQ_BM - 1) / KQ_BM;
   const int mt = blockIdx.x % mtiles;
   const int split = (blockIdx.x / mtiles) % p.splits, strip = blockIdx.x / (mtiles * p.splits);
-  const int cp = strip * 2 + wn;               // column pair of this wavefront
+  const int cp = (p.strip0 + strip) * 2 + wn;  // column pair of this wavefront (strip0: first 256-column strip of the launch)
   const bool wave_on = cp * 128 < p.N;         // N not a multiple of 256: the trailing wavefronts only help staging
   const int row0 = mt * KQ_BM;
 
@@ -81,13 +86,13 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   const int per_q = p.ksteps_per_split / KQ_Q;  // host: a multiple of 4, and the splits are equally long
   const int ks_b = split * p.ksteps_per_split + q * per_q, ks_e = ks_b + per_q;
 
-  // ---- activation staging: the quarter's 128 threads; thread tq loads piece (tq & 7) of tile rows (tq >> 3) + 16 i
+  // ---- activation staging: the K part's 128 threads; thread tq loads piece (tq & 7) of tile rows (tq >> 3) + 16 i
   // (rows without a source read row 0 of A; their results are never stored)
   const int tq = wn * 64 + lane;
   const int piece = tq & 7;
-  const uint16_t* arow[4];
+  const uint16_t* arow[KQ_MB];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < KQ_MB; ++i) {
     int src, dst;
     tile_row_ids((tq >> 3) + 16 * i, src, dst);
     arow[i] = (const uint16_t*)p.A + (int64_t)(src < 0 ? 0 : src) * p.lda + piece * 8;
@@ -95,24 +100,24 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   // LDS A layout per quarter: [buffer][k-step 2][m-block 4][lane 64][4 dwords]; the 16 bytes of (row, piece) are the
   // K pairs 8*pp + 2j (pp = piece & 3), which belong to lane (j*16 + row%16), dword pp, of k-step piece >> 2.
   uint32_t* lds = (uint32_t*)smem + q * (2 * KQ_ABUF / 4);
-  int a_wr[4];
+  int a_wr[KQ_MB];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < KQ_MB; ++i) {
     const int r = (tq >> 3) + 16 * i;
     a_wr[i] = (((piece >> 2) * KQ_MB + (r >> 4)) * 64 + (r & 15)) * 4 + (piece & 3);
   }
-  u32x4 areg[4];
+  u32x4 areg[KQ_MB];
   // (chunk and k-step indices are clamped instead of guarded: the last iteration re-reads its own data, which
   //  keeps the main loop free of branches)
   auto load_a = [&](int chunk) {  // chunk: relative to ks_b
     chunk = min(ks_b / 2 + chunk, ks_e / 2 - 1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
+    for (int i = 0; i < KQ_MB; ++i) areg[i] = *(const u32x4*)(arow[i] + chunk * 64);
   };
   auto store_a = [&](int buf) {
     uint32_t* dst = lds + buf * (KQ_ABUF / 4);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < KQ_MB; ++i) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) dst[a_wr[i] + j * 64] = areg[i][j];
     }
@@ -159,16 +164,21 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   store_a(0);
   // B operands of two Marlin words: the one whose MFMAs are being issued and the one being dequantised
   u32x4 ob[2][2];
-  {
-    const ColConst<DT> cc = col_const(st[0], 0);
-    dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], cc, ob[0][0], ob[0][1]);
-  }
+  // dequantisation constants of the four word positions for the k-step whose operands are being built.  A loop iteration
+  // covers four k-steps (128 rows of K, aligned: every K part starts at a multiple of four k-steps), so with groups of
+  // 128 rows or more, or one scale per column, they are rebuilt once per iteration instead of once per k-step.
+  // (128-row tiles only: with two wavefronts per SIMD the 64-row tiles have no registers to spare for them.)
+  constexpr bool HOIST = (KQ_MB == 8);
+  ColConst<DT> ccs[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) ccs[w] = col_const(st[0], w);
+  dequant_pair<DT, UNIT>(st[0].b0[0], st[0].b1[0], ccs[0], ob[0][0], ob[0][1]);
   __syncthreads();
 
-  // One k-step: per Marlin word w, 8 MFMAs on ob[w & 1]; after each MFMA one register of the following word's
+  // One k-step: per Marlin word w, 2 MB MFMAs on ob[w & 1]; after each MFMA (MB = 8: pair of MFMAs) one register of the following word's
   // operands (word w + 1 of this k-step, or word 0 of the next k-step `nxt`) is dequantised into ob[(w + 1) & 1].
   // The scheduling barriers keep the compiler from regrouping this into MFMA-only and VALU-only blocks.
-  auto kstep = [&](int buf, int kk, const Stage& cur, const Stage& nxt) {
+  auto kstep = [&](int buf, int kk, const Stage& cur, const Stage& nxt, auto refresh_tag) {
     const u32x4* abase = (const u32x4*)(lds + buf * (KQ_ABUF / 4)) + (kk * KQ_MB) * 64 + lane;
     u32x4 af[KQ_MB];
 #pragma unroll
@@ -177,11 +187,23 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
       constexpr int w = decltype(w_tag)::value;
       constexpr int wn2 = (w + 1) & 3;
       const Stage& src = w == 3 ? nxt : cur;
-      const ColConst<DT> cc = col_const(src, wn2);
+      ColConst<DT> cc_word;
+      if constexpr (!HOIST) {
+        cc_word = col_const(src, wn2);
+      } else if constexpr (w == 3 && decltype(refresh_tag)::value) {  // the words of `cur` are done: constants of `nxt`
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) ccs[ww] = col_const(nxt, ww);
+      }
+      const ColConst<DT>& cc = HOIST ? ccs[wn2] : cc_word;
       const uint32_t xa = src.b0[wn2], xb = src.b1[wn2];
       auto step = [&](auto j_tag) {
         constexpr int J = decltype(j_tag)::value;
-        mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
+        if constexpr (KQ_MB == 4) {
+          mfma_inplace<DT>(acc[J >> 1][w][J & 1], af[J >> 1], ob[w & 1][J & 1]);
+        } else {
+          mfma_inplace<DT>(acc[J][w][0], af[J], ob[w & 1][0]);
+          mfma_inplace<DT>(acc[J][w][1], af[J], ob[w & 1][1]);
+        }
         const uint32_t r = dequant_piece<DT, UNIT, J>(xa, xb, cc);
         if constexpr (J < 4)
           ob[wn2 & 1][0][J] = r;
@@ -204,24 +226,37 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
     word(std::integral_constant<int, 3>{});
   };
 
-  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration; all quarters run the same count
+  // ---- main loop: two chunks (four k-steps = the weight ring) per iteration; all K parts run the same count.  The
+  // last k-step of an iteration builds the first operands of the next 128 rows of K: the constants are rebuilt there,
+  // and in the other three k-steps too when a group is shorter than 128 rows.
+  auto main_loop = [&](auto every_tag) {
+    const std::true_type refresh{};
 #pragma unroll 1
-  for (int c0 = 0; c0 < nchunks; c0 += 2) {
-    const int ks0 = 2 * c0;
-    load_a(c0 + 1);
-    kstep(0, 0, st[0], st[1]);
-    issue(st[0], ks0 + 4);
-    kstep(0, 1, st[1], st[2]);
-    issue(st[1], ks0 + 5);
-    store_a(1);
-    __syncthreads();
-    load_a(c0 + 2);
-    kstep(1, 0, st[2], st[3]);
-    issue(st[2], ks0 + 6);
-    kstep(1, 1, st[3], st[0]);
-    issue(st[3], ks0 + 7);
-    store_a(0);
-    __syncthreads();
+    for (int c0 = 0; c0 < nchunks; c0 += 2) {
+      const int ks0 = 2 * c0;
+      load_a(c0 + 1);
+      kstep(0, 0, st[0], st[1], every_tag);
+      issue(st[0], ks0 + 4);
+      kstep(0, 1, st[1], st[2], every_tag);
+      issue(st[1], ks0 + 5);
+      store_a(1);
+      __syncthreads();
+      load_a(c0 + 2);
+      kstep(1, 0, st[2], st[3], every_tag);
+      issue(st[2], ks0 + 6);
+      kstep(1, 1, st[3], st[0], refresh);
+      issue(st[3], ks0 + 7);
+      store_a(0);
+      __syncthreads();
+    }
+  };
+  if constexpr (CHANNEL || !HOIST) {
+    main_loop(std::false_type{});
+  } else {
+    if (p.group_shift < 2)
+      main_loop(std::true_type{});
+    else
+      main_loop(std::false_type{});
   }
 
   // ------------------------------------------------------------------------------ epilogue
@@ -229,7 +264,7 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
   //  accumulators are read)
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   // per m-block: every wavefront writes its 16 x 128 partial to its slab [16 rows][RED_RS]; after a barrier the
-  // wavefront of quarter q adds the four quarters' slabs of its column pair for rows 4q .. 4q+3 and finishes them.
+  // wavefront of K part q adds the Q parts' slabs of its column pair for rows (16 / Q) q .. and finishes them.
   // (the last barrier of the loop separates the slabs from the A buffers they overlay)
   float* slabs = (float*)smem;
   float* mine = slabs + wv * (16 * RED_RS);
@@ -262,8 +297,8 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
         for (int r = 0; r < 4; ++r) mine[(4 * g + r) * RED_RS + 72 * h + 16 * w + 8 * hf + c] = acc[mb][w][hf][r];
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int r16 = 4 * q + (lane >> 5) + 2 * i;
+    for (int i = 0; i < 8 / KQ_Q; ++i) {
+      const int r16 = (16 / KQ_Q) * q + (lane >> 5) + 2 * i;
       const int crow = s_crow[mb * 16 + r16];
       f32x4 v = {0, 0, 0, 0};
 #pragma unroll
@@ -289,14 +324,15 @@ __global__ __launch_bounds__(512) void kq_kernel(const KParams p) {
 
 // Second pass of a split-K launch: adds the splits' partial tiles in split order, then channel scale, bias and
 // conversion as kq_kernel's own epilogue.  One workgroup per (tile, 16-row block); thread -> 4 columns of 4 rows.
-template <int DT, bool CHANNEL>
+template <int DT, bool CHANNEL, int MB = 4>
 __global__ __launch_bounds__(256) void kq_reduce_kernel(const KParams p) {
+  constexpr int KQ_BM = 16 * MB;
   const int t = threadIdx.x;
   const int mtiles = (p.M + KQ_BM - 1) / KQ_BM;
-  const int tile = blockIdx.x >> 2, rb = blockIdx.x & 3;
+  const int tile = blockIdx.x / MB, rb = blockIdx.x % MB;
   const int mt = tile % mtiles, strip = tile / mtiles;
   const int fc4 = (t & 63) * 4;
-  const int ncol = strip * KQ_TN + fc4;
+  const int ncol = (p.strip0 + strip) * KQ_TN + fc4;
   if (ncol >= p.N) return;
   const uint16_t* Sc = (const uint16_t*)p.S;
   const uint16_t* bias = (const uint16_t*)p.bias;
@@ -336,28 +372,37 @@ __global__ __launch_bounds__(256) void kq_reduce_kernel(const KParams p) {
 
 typedef void (*kq_fn)(const KParams);
 
-template <int DT>
+template <int DT, int MB, int Q>
 static kq_fn pick_kq(bool zp, bool channel) {
-  if (zp) return channel ? kq_kernel<DT, true, true> : kq_kernel<DT, true, false>;
-  return channel ? kq_kernel<DT, false, true> : kq_kernel<DT, false, false>;
+  if (zp) return channel ? kq_kernel<DT, true, true, MB, Q> : kq_kernel<DT, true, false, MB, Q>;
+  return channel ? kq_kernel<DT, false, true, MB, Q> : kq_kernel<DT, false, false, MB, Q>;
+}
+template <int DT, int MB>
+static kq_fn pick_kq_reduce(bool channel) {
+  return channel ? kq_reduce_kernel<DT, true, MB> : kq_reduce_kernel<DT, false, MB>;
 }
 
 int launch_kq(const w4a16_gemm_args* a, const Plan& pl, hipStream_t stream) {
   const bool zp = a->b_zeros != nullptr, channel = pl.gm == GM_CHANNEL;
+  const bool tall = pl.mb == 8;  // 128 x 256 tiles with K in halves; otherwise 64 x 256 with K in quarters
+  const int parts = tall ? 2 : 4;
   if ((a->wtype != W4A16_WTYPE_U4B8 && a->wtype != W4A16_WTYPE_U4) || (a->flags & (W4A16_F_ZP_FLOAT | W4A16_F_MOE)) ||
-      pl.gm == GM_GIDX || pl.use_perm || pl.splits < 1 || pl.kps * pl.splits != pl.total_ksteps || pl.kps % 16 != 0 ||
-      pl.tn != KQ_TN)
+      pl.gm == GM_GIDX || pl.use_perm || pl.splits < 1 || pl.kps * pl.splits != pl.total_ksteps ||
+      pl.kps % (4 * parts) != 0 || pl.tn != KQ_TN || (pl.mb != 4 && pl.mb != 8))
     return fail(W4A16_EINVAL, "unsupported kernel variant");
-  const kq_fn fn = a->dtype == DT_F16 ? pick_kq<DT_F16>(zp, channel) : pick_kq<DT_BF16>(zp, channel);
+  const bool f16 = a->dtype == DT_F16;
+  const kq_fn fn = tall ? (f16 ? pick_kq<DT_F16, 8, 2>(zp, channel) : pick_kq<DT_BF16, 8, 2>(zp, channel))
+                        : (f16 ? pick_kq<DT_F16, 4, 4>(zp, channel) : pick_kq<DT_BF16, 4, 4>(zp, channel));
+  const int smem = tall ? kq_smem(8, 2) : kq_smem(4, 4);
   KParams p = make_kparams(a, pl);
   if (pl.tiles <= 0) return 0;
-  W4A16_HIP(allow_dynamic_lds((const void*)fn, KQ_SMEM));
-  hipLaunchKernelGGL(fn, dim3((unsigned)((int64_t)pl.tiles * pl.splits)), dim3(512), KQ_SMEM, stream, p);
+  W4A16_HIP(allow_dynamic_lds((const void*)fn, smem));
+  hipLaunchKernelGGL(fn, dim3((unsigned)((int64_t)pl.tiles * pl.splits)), dim3(128 * parts), smem, stream, p);
   W4A16_HIP(hipGetLastError());
   if (pl.splits > 1) {
-    const kq_fn red = a->dtype == DT_F16 ? (channel ? kq_reduce_kernel<DT_F16, true> : kq_reduce_kernel<DT_F16, false>)
-                                         : (channel ? kq_reduce_kernel<DT_BF16, true> : kq_reduce_kernel<DT_BF16, false>);
-    hipLaunchKernelGGL(red, dim3((unsigned)pl.tiles * 4), dim3(256), 0, stream, p);
+    const kq_fn red = tall ? (f16 ? pick_kq_reduce<DT_F16, 8>(channel) : pick_kq_reduce<DT_BF16, 8>(channel))
+                           : (f16 ? pick_kq_reduce<DT_F16, 4>(channel) : pick_kq_reduce<DT_BF16, 4>(channel));
+    hipLaunchKernelGGL(red, dim3((unsigned)pl.tiles * pl.mb), dim3(256), 0, stream, p);
     W4A16_HIP(hipGetLastError());
   }
   return 0;
