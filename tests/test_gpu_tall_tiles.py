@@ -76,3 +76,38 @@ def test_tall_tiles_one_hot_rows_are_exact(ops, dev, workspace, m, k, n, dtype, 
     out = run_gemm(ops, layer, a.to(dev), dev, workspace)
     torch.cuda.synchronize()
     assert torch.equal(out.cpu(), layer.w_ref[ks])
+
+
+def _random_tall_shapes(count, seed):
+    """Shapes whose 128 x 256 tiles number between 192 and 256: ragged last row tile, last strip 64..256 columns wide."""
+    import random
+    rng = random.Random(seed)
+    out = []
+    while len(out) < count:
+        rows, strips = rng.randint(2, 32), rng.randint(6, 128)
+        if not 192 <= rows * strips <= 256:
+            continue
+        m = 128 * (rows - 1) + rng.randint(1, 128)
+        n = 256 * (strips - 1) + 64 * rng.randint(1, 4)
+        k = 256 * rng.randint(1, 5)
+        mode = rng.choice(["gptq", "awq", "act_order"])
+        group = rng.choice([32, 64, 128] if mode == "act_order" else [-1, 32, 64, 128])
+        out.append((m, k, n, mode, group, rng.choice([torch.float16, torch.bfloat16]), rng.random() < 0.5))
+    return out
+
+
+@pytest.mark.parametrize("cfg", _random_tall_shapes(12, 4242), ids=lambda c: f"m{c[0]}-k{c[1]}-n{c[2]}-{c[3]}-g{c[4]}-"
+                         f"{'f16' if c[5] == torch.float16 else 'bf16'}{'-strided' if c[6] else ''}")
+def test_tall_tiles_random_shapes(ops, dev, workspace, cfg):
+    m, k, n, mode, group, dtype, strided = cfg
+    print(f"tall tiles random {cfg}", flush=True)
+    layer = make_layer(k, n, group, dtype, has_zp=mode == "awq", act_order=mode == "act_order", seed=m + n + k, w_std=0.05)
+    g = torch.Generator().manual_seed(m * 3 + n)
+    if strided:  # a column slice of a wider tensor: rows are k + 64 elements apart
+        a = torch.randn(m, k + 64, generator=g).to(dtype).to(dev)[:, 32:32 + k]
+    else:
+        a = torch.randn(m, k, generator=g).to(dtype).to(dev)
+    out = run_gemm(ops, layer, a, dev, workspace)
+    torch.cuda.synchronize()
+    check_close(out.cpu(), a.contiguous().cpu(), layer)
+    assert int(workspace.abs().sum()) == 0
