@@ -37,6 +37,8 @@ CASES = [
     (2048, 16384, 128, torch.float16, False, False, (256, 200)),  # 64-row kernel, two-pass K split (32 MiB of partials)
     (2048, 1024, 128, torch.float16, False, True, (40, 5)),       # act-order: A gathered into the scratch
     (4096, 6144, 128, torch.bfloat16, True, False, (300, 130)),   # prefill kernel (no scratch needed)
+    (1024, 4096, 128, torch.bfloat16, True, False, (2048, 1600)), # 128 x 256 tiles, K halves inside the workgroup
+    (512, 6144, 128, torch.float16, False, False, (4096, 4000)),  # prefill kernel + 128 x 256 tiles on the last strips
 ]
 
 
