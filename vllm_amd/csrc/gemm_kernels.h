@@ -30,7 +30,7 @@ struct KParams {
   int splits, ksteps_per_split, total_ksteps;
   int xcd_map;
   int tn;        // tile width in columns (128, or 64 for the narrow decode tiles)
-  int strip0;    // 64-row kernel: first 512-column strip of this launch (it may finish what the prefill kernel left)
+  int strip0;    // 64-row kernel / K-split kernel: first 512- / 256-column strip of this launch (it may finish what the prefill kernel left)
   int dyn_slots; // 64-row kernel, MoE: > 0 = the K split is chosen on the device from the number of live blocks (tail_split)
   // MoE
   const int32_t* sorted_ids;

@@ -1,6 +1,6 @@
-// W4A16 GEMM for gfx950 with 64-row tiles and an in-workgroup K split: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias),
-// dense, for 33..128 rows and wide N, where the 64 x 512 tiles of the 64-row kernel are too few to fill the chip
-// (the reference's small-batch thread configurations, csrc/quantization/gptq_marlin/gptq_marlin.cu:120-170).
+// W4A16 GEMM for gfx950 with an in-workgroup K split: C[M,N] = A[M,K] * dequant(Bq)[K,N] (+bias), dense, in two shapes.
+// First shape, 64-row tiles: 33..128 rows and wide N, where the 64 x 512 tiles of the 64-row kernel are too few to fill
+// the chip (the reference's small-batch thread configurations, csrc/quantization/gptq_marlin/gptq_marlin.cu:120-170).
 //
 //   workgroup tile 64 rows x 256 columns, 8 wavefronts = 2 column pairs x 4 K-quarters: every wavefront owns
 //   64 rows x 128 columns (32 v_mfma_f32_16x16x32 per k-step, 128 fp32 accumulators in AGPRs) over a quarter of the
@@ -20,9 +20,12 @@
 // A second shape of the same kernel (MB = 8, Q = 2: 4 wavefronts, one per SIMD, 128 rows x 256 columns, K in halves, 256
 // accumulators per lane) serves problems with 128-row tiles that are too few for the prefill kernel's 128 x 512 tiles:
 // every dequantised operand register feeds eight row blocks as in the prefill kernel, and the two K halves are added
-// through LDS instead of through memory.
-// Requirements (host-checked): K % 512 == 0 (Q = 2: K % 256 == 0) (every quarter runs whole ring periods of 4 k-steps), scales grouped (a
-// power-of-two number of k-steps) or channelwise, no per-row g_idx, A's columns already in weight order.
+// through LDS instead of through memory.  The host uses it for more than 128 rows when these tiles fill 3/4 to all of the
+// compute units in one round, and for the trailing strips of a prefill launch whose last round is at most half full
+// (KParams.strip0: first 256-column strip of the launch).
+// Requirements (host-checked): K % 512 == 0 (second shape: K % 256 == 0), so that every K part runs whole ring periods of
+// 4 k-steps; scales grouped (a power-of-two number of k-steps) or channelwise, no per-row g_idx, A's columns already in
+// weight order.
 #include <type_traits>
 
 #include "gemm_kernels.h"

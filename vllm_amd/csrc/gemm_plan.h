@@ -17,7 +17,7 @@ struct Plan {
              // 5: in-workgroup K split (gemm_kq.hip): 64 x 256 tiles in K quarters (mb = 4), 128 x 256 in halves (mb = 8)
   int tn;    // tile width in columns (128; the decode kernel also has 64)
   int nw = 8;  // 16-row tiles (decode kernel, general kernel with one m-block): wavefronts per workgroup (8 or 4)
-  int strip0 = 0;      // 64-row kernel: first 512-column strip handled by the launch
+  int strip0 = 0;      // 64-row kernel / K-split kernel: first 512- / 256-column strip handled by the launch
   int dyn_slots = 0;   // 64-row kernel, MoE: resident workgroups that the device-side K split of the tail tiles fills
   int tail_strips = 0; // prefill plan: trailing 512-column strips handed to another kernel (0 = none)
   int tail_kind = 3;   // ... which one: 3 = 64-row kernel, 5 = 128 x 256 tiles with the K halves inside the workgroup
